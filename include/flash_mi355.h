@@ -1,0 +1,150 @@
+/*
+ * flash_mi355.h -- C ABI of the MI355X (gfx950) flexible-mask flash-attention library.
+ *
+ * One shared library, plain pointers and sizes, no torch or HIP types in any
+ * signature (a HIP stream is passed as void*).  The library allocates nothing,
+ * keeps no state between calls and never synchronises the host: every entry
+ * point enqueues kernels on the caller's stream and returns.
+ *
+ * Each entry point replaces one launch site of the reference operator
+ * (flash_triton.py of zzsfornlp/Triton-Flash-Attention-with-Flexible-Masks):
+ *
+ *   fa_fwd        <- _fwd_kernel[grid](...)          flash_triton.py:541-556
+ *   fa_bwd_delta  <- _bwd_preprocess[grid](...)      flash_triton.py:585-592
+ *   fa_bwd_dkdv   <- _bwd_kv_kernel[grid](...)       flash_triton.py:596-614
+ *   fa_bwd_dq     <- _bwd_q_kernel[grid](...)        flash_triton.py:617-634
+ *   fa_mask_plan  <- (no counterpart: the reference evaluates the doc mask on
+ *                     every tile, README.md:18)  builds the per-tile id
+ *                     summaries the kernels use to skip fully masked tiles
+ *   fa_mask_dump  <- the mask expression of flash_triton.py:103-116 written out
+ *                     as bytes, for bit-exact mask tests
+ *   fa_validate   <- the asserts of FlashAttention.forward, flash_triton.py:508-530
+ *
+ * Tensor conventions (identical to the reference, flash_triton.py:27-36):
+ *   q, o, dout, dq : [B, H,  M, D]      k, v : [B, Hk, N, D]   (H % Hk == 0)
+ *   dk, dv         : [B, H,  N, D]      per *query* head (flash_triton.py:594-595);
+ *                                       the caller sums over the group when Hk < H
+ *   lse, delta     : [B, H, M] float32, contiguous.  lse is in log2 units
+ *                    (m + log2(l), flash_triton.py:133); -inf for a row with
+ *                    no unmasked key
+ *   eq : [B, H, M]   ek : [B, H, N]     integer ids, indexed by the *query* head
+ *                                       (flash_triton.py:75-76), any strides
+ *                                       including 0
+ * Strides are in elements.  The innermost stride of every 4-D tensor must be 1
+ * (the reference forces that with maybe_contiguous, flash_triton.py:435-437,525).
+ * Base pointers must be 16-byte aligned and row strides multiples of 8 elements.
+ */
+#ifndef FLASH_MI355_H
+#define FLASH_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_ABI_VERSION 1
+
+/* score_func_mode, flash_triton.py:20-22 */
+#define FA_SCORE_MODE0_NOPE 0
+#define FA_SCORE_MODE1_DOC  1
+
+/* element types */
+#define FA_DTYPE_BF16 0
+#define FA_DTYPE_FP16 1
+#define FA_IDTYPE_I32 0
+#define FA_IDTYPE_I64 1
+
+/* return codes */
+#define FA_OK                    0
+#define FA_ERR_NULLPTR          -1
+#define FA_ERR_UNSUPPORTED_D    -2   /* D not in {16,32,64,128}: flash_triton.py:512 */
+#define FA_ERR_DTYPE            -3
+#define FA_ERR_SHAPE            -4   /* H % Hk != 0, causal with N < M, sizes <= 0 */
+#define FA_ERR_ALIGN            -5
+#define FA_ERR_STRIDE           -6
+#define FA_ERR_MODE             -7   /* unknown score mode, or doc mode without ids */
+#define FA_ERR_WORKSPACE        -8   /* workspace missing or too small */
+#define FA_ERR_HIP              -9   /* kernel launch failed; see fa_last_hip_error */
+#define FA_ERR_NOT_IMPLEMENTED -10
+
+typedef struct fa_params {
+  /* forward operands */
+  const void* q;
+  const void* k;
+  const void* v;
+  void*       o;
+  float*      lse;        /* [B,H,M] log2-domain */
+  /* backward operands */
+  const void* dout;
+  void*       dq;
+  void*       dk;         /* [B,H,N,D] */
+  void*       dv;         /* [B,H,N,D] */
+  float*      delta;      /* [B,H,M] */
+  /* flexible-mask ids */
+  const void* eq;
+  const void* ek;
+  /* scratch written by fa_mask_plan and read by the compute kernels
+     (required when score_mode != 0; size from fa_workspace_bytes) */
+  void*       workspace;
+  uint64_t    workspace_bytes;
+
+  int64_t q_stride[4], k_stride[4], v_stride[4], o_stride[4];
+  int64_t do_stride[4], dq_stride[4], dk_stride[4], dv_stride[4];
+  int64_t eq_stride[3], ek_stride[3];
+
+  int32_t B, H, Hk, M, N, D;
+  int32_t causal;         /* bottom-right aligned: keep iff max(0,N-M)+i >= j */
+  int32_t score_mode;     /* FA_SCORE_MODE* */
+  int32_t dtype;          /* FA_DTYPE_*  (q,k,v,o,dout,dq,dk,dv share it) */
+  int32_t id_dtype;       /* FA_IDTYPE_* (eq, ek) */
+  float   sm_scale;
+  int32_t flags;          /* reserved, must be 0 */
+} fa_params;
+
+/* ABI version of the loaded library (== FA_ABI_VERSION of the header it was built from). */
+int fa_version(void);
+
+/* sizeof(fa_params) as compiled, so a binding can check its own struct packing. */
+uint64_t fa_params_size(void);
+
+/* Static text for a return code. */
+const char* fa_error_string(int code);
+
+/* hipError_t of the last failed launch on this thread (0 if none). */
+int fa_last_hip_error(void);
+
+/* Shape / dtype / stride / alignment / null checks for the given stage.
+   Touches no GPU API; callable on a machine without a GPU.
+   stage: 0 = forward, 1 = backward (all three backward kernels), 2 = mask plan only. */
+int fa_validate(const fa_params* p, int stage);
+
+/* Bytes of workspace fa_mask_plan needs for these sizes (0 when score_mode == 0). */
+uint64_t fa_workspace_bytes(const fa_params* p);
+
+/* Mask engine: normalise eq/ek to int32 and build per-tile id summaries
+   into p->workspace.  Must be enqueued before fa_fwd / fa_bwd_* on the same
+   stream whenever score_mode != 0.  The same workspace serves forward and backward. */
+int fa_mask_plan(const fa_params* p, void* stream);
+
+/* O = softmax(q k^T * sm_scale + mask) v ; lse = log2-sum-exp2 of the scaled scores. */
+int fa_fwd(const fa_params* p, void* stream);
+
+/* delta = rowsum(o * dout). */
+int fa_bwd_delta(const fa_params* p, void* stream);
+
+/* dk, dv per query head (needs lse, delta). */
+int fa_bwd_dkdv(const fa_params* p, void* stream);
+
+/* dq (needs lse, delta). */
+int fa_bwd_dq(const fa_params* p, void* stream);
+
+/* Write keep(i,j) as one byte (0/1) per element into out[B,H,M,N] (contiguous),
+   evaluated by the same device routine the compute kernels use. */
+int fa_mask_dump(const fa_params* p, uint8_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_MI355_H */

@@ -1,0 +1,129 @@
+"""GPU parity: the HIP operator (through the C ABI) against the CPU oracle on the
+same seeded inputs.  Tolerances (bf16/fp16 inputs, fp32 oracle on the same
+rounded inputs): O, dQ, dK, dV max-abs <= 2e-2; LSE max-abs <= 1e-3; mask bit-exact.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL_O = 2e-2
+TOL_LSE = 1e-3
+
+
+def _ids(rng, B, H, L, kind):
+    from flash_mi355 import workloads as W
+    if kind == "uniform":
+        ids = np.stack([W.doc_ids_uniform(rng, L, 8, 96, 0.08) for _ in range(B)])
+    elif kind == "allglobal":
+        ids = np.zeros((B, L), np.int32)
+    elif kind == "alllocal":
+        ids = np.stack([W.doc_ids_uniform(rng, L, 8, 96, 0.0) for _ in range(B)])
+    else:
+        raise KeyError(kind)
+    return ids
+
+
+def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
+              id_dtype=torch.int32, sm_scale=None, check_bwd=True):
+    from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    q = torch.randn(B, H, M, D, generator=g).to(dtype)
+    k = torch.randn(B, Hk, N, D, generator=g).to(dtype)
+    v = torch.randn(B, Hk, N, D, generator=g).to(dtype)
+    do = torch.randn(B, H, M, D, generator=g).to(dtype)
+    eq = ek = None
+    mode = 0
+    if doc:
+        mode = SCORE_FUNC_MODE1_DOC
+        if per_head_ids:
+            ekn = np.stack([_ids(rng, B, H, N, ids_kind) for _ in range(H)], axis=1)  # [B,H,N]
+            ek = torch.from_numpy(ekn).to(id_dtype)
+        else:
+            ek = torch.from_numpy(_ids(rng, B, H, N, ids_kind)).to(id_dtype)[:, None, :].expand(B, H, N)
+        eq = ek[:, :, N - M:]  # queries are the last M positions (self-attention when M == N)
+    print(f"case B{B} H{H}/{Hk} M{M} N{N} D{D} {dtype} causal={causal} doc={doc} seed={seed} ids={ids_kind}", flush=True)
+
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    eqd = eq.cuda() if eq is not None else None
+    ekd = ek.cuda() if ek is not None else None
+    if eqd is not None and not per_head_ids:
+        eqd = eq[:, :1].contiguous().cuda().expand(B, H, M)
+        ekd = ek[:, :1].contiguous().cuda().expand(B, H, N)
+    out, lse = attention_with_lse(qd.detach(), kd.detach(), vd.detach(), causal, sm_scale, eqd, ekd, mode)
+    torch.cuda.synchronize()
+    ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, sm_scale, eq, ek, mode)
+    # rows without any kept key: O = 0, LSE = -inf on both sides
+    dead = torch.isinf(ref_lse)
+    assert torch.equal(torch.isinf(lse.cpu()), dead)
+    lse_err = (lse.cpu()[~dead] - ref_lse[~dead]).abs().max().item() if (~dead).any() else 0.0
+    o_err = (out.float().cpu() - ref_o).abs().max().item()
+    assert not torch.isnan(out).any()
+    assert lse_err <= TOL_LSE, f"LSE err {lse_err}"
+    assert o_err <= TOL_O, f"O err {o_err}"
+    if not check_bwd:
+        return
+    out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode)
+    out2.backward(do.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(out2.detach(), out)
+    for name, got, ref in (("dq", qd.grad, ref_dq), ("dk", kd.grad, ref_dk), ("dv", vd.grad, ref_dv)):
+        assert got.shape == ref.shape, name
+        assert not torch.isnan(got).any(), name
+        err = (got.float().cpu() - ref).abs().max().item()
+        # the gradient itself is rounded to bf16/fp16 on output: half an ulp at magnitude x
+        # is x * 2^-9, so the absolute bound grows with the gradient's magnitude above 4
+        scale = max(1.0, ref.abs().max().item() / 4)
+        assert err <= TOL_O * scale, f"{name} err {err} (ref max {ref.abs().max().item()})"
+
+
+CASES = [
+    # B, H, Hk, M, N, D, dtype, causal, doc
+    (1, 2, 2, 128, 128, 128, torch.bfloat16, False, False),
+    (1, 2, 2, 256, 256, 128, torch.bfloat16, True, False),
+    (2, 2, 2, 256, 256, 128, torch.bfloat16, True, True),
+    (1, 2, 2, 384, 384, 64, torch.bfloat16, True, True),
+    (1, 2, 2, 256, 256, 64, torch.float16, False, True),
+    (1, 4, 2, 256, 256, 128, torch.bfloat16, True, True),      # grouped-query
+    (1, 2, 2, 128, 512, 128, torch.float16, True, True),       # rectangular, bottom-right causal
+    (1, 2, 2, 200, 200, 128, torch.bfloat16, True, True),      # ragged lengths
+    (1, 2, 2, 77, 333, 64, torch.bfloat16, True, True),        # ragged + rectangular
+    (1, 2, 2, 256, 256, 32, torch.bfloat16, True, True),
+    (1, 1, 1, 1024, 1024, 128, torch.bfloat16, True, True),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d-H%d_%d-M%d-N%d-D%d-%s-c%d-d%d" % (
+    c[0], c[1], c[2], c[3], c[4], c[5], str(c[6]).split(".")[-1], c[7], c[8]))
+def test_fwd_bwd_parity(case):
+    _run_case(*case, seed=1234)
+
+
+def test_mask_bit_exact():
+    from flash_mi355 import mask_dump, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    rng = np.random.default_rng(7)
+    for (B, H, M, N, causal) in [(2, 3, 200, 200, True), (1, 2, 77, 333, True), (1, 2, 130, 64, False)]:
+        ek = torch.from_numpy(np.stack([_ids(rng, B, H, N, "uniform") for _ in range(H)], axis=1))
+        eq = torch.from_numpy(np.stack([_ids(rng, B, H, M, "uniform") for _ in range(H)], axis=1))
+        for idt in (torch.int32, torch.int64):
+            got = mask_dump(B, H, M, N, causal, eq.to(idt).cuda(), ek.to(idt).cuda(), SCORE_FUNC_MODE1_DOC).cpu().numpy()
+            ref = np.broadcast_to(O.keep_mask(M, N, causal, eq.numpy(), ek.numpy(), 1), (B, H, M, N))
+            assert np.array_equal(got, ref)
+        got = mask_dump(B, H, M, N, causal).cpu().numpy()
+        ref = np.broadcast_to(O.keep_mask(M, N, causal), (B, H, M, N))
+        assert np.array_equal(got, ref)
+
+
+def test_all_global_and_all_local_ids():
+    _run_case(1, 2, 2, 256, 256, 128, torch.bfloat16, True, True, seed=5, ids_kind="allglobal")
+    _run_case(1, 2, 2, 256, 256, 128, torch.bfloat16, True, True, seed=6, ids_kind="alllocal")
+
+
+def test_per_head_int64_ids():
+    _run_case(1, 3, 3, 192, 192, 64, torch.bfloat16, True, True, seed=9, per_head_ids=True, id_dtype=torch.int64)

@@ -1,0 +1,162 @@
+// C ABI of the library (see include/flash_mi355.h): argument validation that
+// mirrors the asserts of FlashAttention.forward (flash_triton.py:508-530),
+// translation of fa_params into the kernel-side view, and dispatch.
+#include "fa_common.h"
+
+using namespace fa;
+
+static thread_local int g_last_hip_error = 0;
+
+static bool d_supported(int D) { return D == 16 || D == 32 || D == 64 || D == 128; }
+
+static int check_tensor(const void* ptr, const int64_t* st) {
+  if (ptr == nullptr) return FA_ERR_NULLPTR;
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0) return FA_ERR_ALIGN;
+  if (st[3] != 1) return FA_ERR_STRIDE;
+  if ((st[0] % 8) != 0 || (st[1] % 8) != 0 || (st[2] % 8) != 0) return FA_ERR_ALIGN;
+  return FA_OK;
+}
+
+extern "C" int fa_version(void) { return FA_ABI_VERSION; }
+extern "C" uint64_t fa_params_size(void) { return sizeof(fa_params); }
+extern "C" int fa_last_hip_error(void) { return g_last_hip_error; }
+
+extern "C" const char* fa_error_string(int code) {
+  switch (code) {
+    case FA_OK: return "ok";
+    case FA_ERR_NULLPTR: return "null pointer for a required operand";
+    case FA_ERR_UNSUPPORTED_D: return "head dimension must be one of 16, 32, 64, 128";
+    case FA_ERR_DTYPE: return "unsupported element or id type";
+    case FA_ERR_SHAPE: return "inconsistent sizes (H % Hk != 0, causal with N < M, or a size <= 0)";
+    case FA_ERR_ALIGN: return "pointers must be 16-byte aligned and outer strides multiples of 8 elements";
+    case FA_ERR_STRIDE: return "innermost stride must be 1";
+    case FA_ERR_MODE: return "unknown score mode, or doc mode without eq/ek";
+    case FA_ERR_WORKSPACE: return "workspace missing or too small";
+    case FA_ERR_HIP: return "kernel launch failed";
+    case FA_ERR_NOT_IMPLEMENTED: return "configuration not implemented";
+    default: return "unknown error";
+  }
+}
+
+extern "C" int fa_validate(const fa_params* p, int stage) {
+  if (p == nullptr) return FA_ERR_NULLPTR;
+  if (!d_supported(p->D)) return FA_ERR_UNSUPPORTED_D;
+  if (p->dtype != FA_DTYPE_BF16 && p->dtype != FA_DTYPE_FP16) return FA_ERR_DTYPE;
+  if (p->B <= 0 || p->H <= 0 || p->Hk <= 0 || p->M <= 0 || p->N <= 0) return FA_ERR_SHAPE;
+  if (p->H % p->Hk != 0) return FA_ERR_SHAPE;
+  if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
+  if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC) return FA_ERR_MODE;
+  if (p->flags != 0) return FA_ERR_MODE;
+  if (p->score_mode == FA_SCORE_MODE1_DOC) {
+    if (p->eq == nullptr || p->ek == nullptr) return FA_ERR_MODE;
+    if (p->id_dtype != FA_IDTYPE_I32 && p->id_dtype != FA_IDTYPE_I64) return FA_ERR_DTYPE;
+    if (p->workspace == nullptr) return FA_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(p->workspace) & 255) != 0) return FA_ERR_ALIGN;
+    if (p->workspace_bytes < fa_workspace_bytes(p)) return FA_ERR_WORKSPACE;
+  }
+  if (stage == 2) return FA_OK;
+  int rc;
+  if ((rc = check_tensor(p->q, p->q_stride)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->k, p->k_stride)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->v, p->v_stride)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->o, p->o_stride)) != FA_OK) return rc;
+  if (p->lse == nullptr) return FA_ERR_NULLPTR;
+  if (stage == 1) {
+    if ((rc = check_tensor(p->dout, p->do_stride)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dq, p->dq_stride)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dk, p->dk_stride)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dv, p->dv_stride)) != FA_OK) return rc;
+    if (p->delta == nullptr) return FA_ERR_NULLPTR;
+  }
+  return FA_OK;
+}
+
+extern "C" uint64_t fa_workspace_bytes(const fa_params* p) {
+  if (p == nullptr || p->score_mode == FA_SCORE_MODE0_NOPE) return 0;
+  if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
+  return ws_layout(p).total;
+}
+
+static KArgs make_args(const fa_params* p) {
+  KArgs a;
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;
+  a.dout = p->dout; a.dq = p->dq; a.dk = p->dk; a.dv = p->dv; a.delta = p->delta;
+  a.q_bs = p->q_stride[0]; a.q_hs = p->q_stride[1]; a.q_rs = p->q_stride[2];
+  a.k_bs = p->k_stride[0]; a.k_hs = p->k_stride[1]; a.k_rs = p->k_stride[2];
+  a.v_bs = p->v_stride[0]; a.v_hs = p->v_stride[1]; a.v_rs = p->v_stride[2];
+  a.o_bs = p->o_stride[0]; a.o_hs = p->o_stride[1]; a.o_rs = p->o_stride[2];
+  a.do_bs = p->do_stride[0]; a.do_hs = p->do_stride[1]; a.do_rs = p->do_stride[2];
+  a.dq_bs = p->dq_stride[0]; a.dq_hs = p->dq_stride[1]; a.dq_rs = p->dq_stride[2];
+  a.dk_bs = p->dk_stride[0]; a.dk_hs = p->dk_stride[1]; a.dk_rs = p->dk_stride[2];
+  a.dv_bs = p->dv_stride[0]; a.dv_hs = p->dv_stride[1]; a.dv_rs = p->dv_stride[2];
+  a.B = p->B; a.H = p->H; a.Hk = p->Hk; a.G = p->H / p->Hk; a.M = p->M; a.N = p->N;
+  a.gap = p->N > p->M ? p->N - p->M : 0;  // flash_triton.py:521
+  a.scale = p->sm_scale;
+  a.scale_log2e = p->sm_scale * kLog2e;
+  a.eq32 = nullptr; a.ek32 = nullptr; a.qsum = nullptr; a.ksum = nullptr;
+  a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
+  a.nQs = a.nKs = 0;
+  if (p->score_mode == FA_SCORE_MODE1_DOC) {
+    const WsLayout w = ws_layout(p);
+    char* ws = reinterpret_cast<char*>(p->workspace);
+    a.eq32 = reinterpret_cast<const int*>(ws + w.off_eq32);
+    a.ek32 = reinterpret_cast<const int*>(ws + w.off_ek32);
+    a.qsum = reinterpret_cast<const IdSummary*>(ws + w.off_qsum);
+    a.ksum = reinterpret_cast<const IdSummary*>(ws + w.off_ksum);
+    a.eq_bs = int64_t(w.Hq1) * w.Mp; a.eq_hs = w.Hq1 == 1 ? 0 : w.Mp;
+    a.ek_bs = int64_t(w.Hk1) * w.Np; a.ek_hs = w.Hk1 == 1 ? 0 : w.Np;
+    a.qs_bs = int64_t(w.Hq1) * w.nQs; a.qs_hs = w.Hq1 == 1 ? 0 : w.nQs;
+    a.ks_bs = int64_t(w.Hk1) * w.nKs; a.ks_hs = w.Hk1 == 1 ? 0 : w.nKs;
+    a.nQs = w.nQs; a.nKs = w.nKs;
+  }
+  return a;
+}
+
+static int finish(int hip_rc) {
+  if (hip_rc == 0) return FA_OK;
+  if (hip_rc < 0) return FA_ERR_NOT_IMPLEMENTED;
+  g_last_hip_error = hip_rc;
+  return FA_ERR_HIP;
+}
+
+extern "C" int fa_mask_plan(const fa_params* p, void* stream) {
+  int rc = fa_validate(p, 2);
+  if (rc != FA_OK) return rc;
+  if (p->score_mode == FA_SCORE_MODE0_NOPE) return FA_OK;
+  return finish(launch_mask_plan(p, ws_layout(p), reinterpret_cast<hipStream_t>(stream)));
+}
+
+extern "C" int fa_fwd(const fa_params* p, void* stream) {
+  int rc = fa_validate(p, 0);
+  if (rc != FA_OK) return rc;
+  return finish(launch_fwd(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
+                           reinterpret_cast<hipStream_t>(stream)));
+}
+
+extern "C" int fa_bwd_delta(const fa_params* p, void* stream) {
+  int rc = fa_validate(p, 1);
+  if (rc != FA_OK) return rc;
+  return finish(launch_bwd_delta(make_args(p), p->dtype, p->D, reinterpret_cast<hipStream_t>(stream)));
+}
+
+extern "C" int fa_bwd_dkdv(const fa_params* p, void* stream) {
+  int rc = fa_validate(p, 1);
+  if (rc != FA_OK) return rc;
+  return finish(launch_bwd_dkdv(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
+                                reinterpret_cast<hipStream_t>(stream)));
+}
+
+extern "C" int fa_bwd_dq(const fa_params* p, void* stream) {
+  int rc = fa_validate(p, 1);
+  if (rc != FA_OK) return rc;
+  return finish(launch_bwd_dq(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
+                              reinterpret_cast<hipStream_t>(stream)));
+}
+
+extern "C" int fa_mask_dump(const fa_params* p, uint8_t* out, void* stream) {
+  int rc = fa_validate(p, 2);
+  if (rc != FA_OK) return rc;
+  if (out == nullptr) return FA_ERR_NULLPTR;
+  return finish(launch_mask_dump(make_args(p), p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC, out,
+                                 reinterpret_cast<hipStream_t>(stream)));
+}

@@ -1,0 +1,254 @@
+// dK/dV kernel of the split backward: 128 keys per workgroup (32 per wave) held
+// in registers, query-side tiles (Q, dO, LSE, delta, eq) streamed through LDS.
+// Replaces _bwd_kv_kernel of the reference (flash_triton.py:175-321).
+//
+//   S    = Q K^T           A = Q rows (LDS),  B = K^T (registers, whole kernel)
+//   dP   = dO V^T          A = dO rows (LDS), B = V^T (registers, whole kernel)
+//   P    = exp2(S*c - L), masked elements -> 0           (flash_triton.py:269-280)
+//   dS   = P * (dP - delta)                              (flash_triton.py:301)
+//   dV^T += dO^T P         A = dO^T via ds_read_b64_tr_b16, B = P from the accumulators
+//   dK^T += Q^T dS         A = Q^T  via ds_read_b64_tr_b16, B = dS
+//   dK   = dK * sm_scale                                 (flash_triton.py:313)
+// In the accumulator layout each lane owns ONE key column and 16 query rows of
+// every 32-row block, so LSE / delta / eq are read as broadcast 16-byte LDS loads.
+// dK, dV are written per query head; the group sum for grouped-query attention is
+// done by the caller (flash_triton.py:635-637).
+#include "fa_tile.h"
+
+namespace fa {
+
+template <typename Tag, int D, bool CAUSAL, bool DOC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void bwd_dkdv_kernel(const KArgs a) {
+  using E = Elem<Tag>;
+  using T = typename E::scalar;
+  using vec8 = typename E::vec8;
+  constexpr int BK = 128, BQ = 64, KS = D / 16, DBN = D / 32;
+  constexpr int TILE_BYTES = BQ * D * 2;
+  constexpr int AUX_OFF = 4 * TILE_BYTES;  // [2 buffers][3 arrays][64] x 4 bytes
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lq = lane & 31, g = lane >> 5;
+
+  const int nKt = (a.N + BK - 1) / BK;
+  const int BH = a.B * a.H;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int bh = (idx / nKt) * 8 + xcd;
+  if (bh >= BH) return;
+  const int kt = idx % nKt;  // causal: the first key tiles see the most query rows
+  const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
+
+  const T* qp = reinterpret_cast<const T*>(a.q) + b * a.q_bs + h * a.q_hs;
+  const T* kp = reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs;
+  const T* vp = reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs;
+  const T* dop = reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs;
+  T* dkp = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + h * a.dk_hs;
+  T* dvp = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + h * a.dv_hs;
+  const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
+  const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+
+  const int n0 = kt * BK;
+  const int nw = n0 + wave * 32;
+  const int key = nw + lq;
+  const int keyc = key < a.N ? key : a.N - 1;
+
+  // K^T, V^T fragments (B operands): lane holds d = 16*ks + 8*g .. +7 of its key row.
+  vec8 kf[KS], vf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    kf[ks] = *reinterpret_cast<const vec8*>(kp + int64_t(keyc) * a.k_rs + ks * 16 + g * 8);
+    vf[ks] = *reinterpret_cast<const vec8*>(vp + int64_t(keyc) * a.v_rs + ks * 16 + g * 8);
+  }
+  const float c = a.scale_log2e;
+
+  int ek_j = 0;
+  int wk_lo = 0, wk_hi = 0;   // id interval of this wave's 32 keys
+  int gk_lo = 0, gk_hi = 0;   // of the workgroup's 128 keys
+  const int* eqp = nullptr;
+  const IdSummary* qsum = nullptr;
+  if (DOC) {
+    ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
+    eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
+    qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
+    const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
+    const IdSummary s0 = ks[n0 / kSumRows];
+    gk_lo = s0.lo; gk_hi = s0.hi;
+    if (n0 / kSumRows + 1 < a.nKs) {
+      const IdSummary s1 = ks[n0 / kSumRows + 1];
+      gk_lo = min(gk_lo, s1.lo); gk_hi = max(gk_hi, s1.hi);
+    }
+    const bool valid = key < a.N;
+    int lo = valid ? ek_j : 0x7fffffff, hi = valid ? ek_j : (int)0x80000000;
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1) {
+      lo = min(lo, __shfl_xor(lo, off));
+      hi = max(hi, __shfl_xor(hi, off));
+    }
+    wk_lo = lo; wk_hi = hi;
+  }
+
+  const int nQtiles = (a.M + BQ - 1) / BQ;
+  const int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
+  TileIter it;
+  it.init(first, nQtiles, qsum, gk_lo, gk_hi, 0, false);
+
+  f32x16 dk[DBN], dv[DBN];
+#pragma unroll
+  for (int db = 0; db < DBN; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+
+  auto load_tile = [&](int tile, int bufi) {
+    const int m0 = tile * BQ;
+    tile_load_async<T, D, BQ, SWZ_ROW>(qp, a.q_rs, m0, a.M, smem + bufi * TILE_BYTES);
+    tile_load_async<T, D, BQ, SWZ_ROW>(dop, a.do_rs, m0, a.M, smem + (2 + bufi) * TILE_BYTES);
+    const int r = m0 + lane < a.M ? m0 + lane : a.M - 1;
+    char* aux = smem + AUX_OFF + bufi * 768;
+    if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
+    if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
+    if (DOC && wave == 2) __builtin_amdgcn_global_load_lds(FA_GLB(eqp + r), FA_LDS(aux + 512), 4, 0, 0);
+  };
+
+  int cur = it.next();
+  int buf = 0;
+  if (cur >= 0) load_tile(cur, 0);
+  while (cur >= 0) {
+    const int nxt = it.next();
+    wait_async_loads();
+    __syncthreads();
+    if (nxt >= 0) load_tile(nxt, buf ^ 1);
+    const char* lqt = smem + buf * TILE_BYTES;
+    const char* ldo = smem + (2 + buf) * TILE_BYTES;
+    const char* aux = smem + AUX_OFF + buf * 768;
+    const int m0 = cur * BQ;
+
+    // wave-level decisions: rows m0..m0+63 against keys nw..nw+31
+    bool skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
+    bool need_mask = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
+    if (DOC) {
+      const IdSummary qs = qsum[cur];
+      skip = skip || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
+      need_mask = need_mask || !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
+    }
+    if (!skip) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec8 qa = frag_row<E, D, SWZ_ROW>(lqt, qb * 32 + lq, 2 * ks + g);
+          s = E::mfma32(qa, kf[ks], s);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec8 da = frag_row<E, D, SWZ_ROW>(ldo, qb * 32 + lq, 2 * ks + g);
+          dp = E::mfma32(da, vf[ks], dp);
+        }
+        // s -> P, dp -> dS for this lane's 16 query rows of the block
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
+          const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
+          const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+          i32x4 eqv = {0, 0, 0, 0};
+          if (DOC && need_mask) eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            float p = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
+            if (need_mask) {
+              const int i = m0 + i0 + t;
+              const bool keep = (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
+              p = keep ? p : 0.f;
+            }
+            s[4 * q4 + t] = p;
+            dp[4 * q4 + t] = p * (dp[4 * q4 + t] - dl[t]);
+          }
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          vec8 pf, dsf;
+#pragma unroll
+          for (int t = 0; t < 8; t += 2) {
+            const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
+            const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
+            pf[t] = pr[0]; pf[t + 1] = pr[1];
+            dsf[t] = dr[0]; dsf[t + 1] = dr[1];
+          }
+#pragma unroll
+          for (int db = 0; db < DBN; ++db) {
+            const vec8 dot = frag_tr<E, D, SWZ_TR>(ldo, 32 * qb + 16 * half, db);
+            dv[db] = E::mfma32(dot, pf, dv[db]);
+          }
+#pragma unroll
+          for (int db = 0; db < DBN; ++db) {
+            const vec8 qtf = frag_tr<E, D, SWZ_TR>(lqt, 32 * qb + 16 * half, db);
+            dk[db] = E::mfma32(qtf, dsf, dk[db]);
+          }
+        }
+      }
+    }
+    cur = nxt;
+    buf ^= 1;
+  }
+
+  if (key < a.N) {
+    T* krow = dkp + int64_t(key) * a.dk_rs;
+    T* vrow = dvp + int64_t(key) * a.dv_rs;
+    const float sc = a.scale;
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const typename E::vec2 k0 = E::cvt2(dk[db][4 * q4 + 0] * sc, dk[db][4 * q4 + 1] * sc);
+        const typename E::vec2 k1 = E::cvt2(dk[db][4 * q4 + 2] * sc, dk[db][4 * q4 + 3] * sc);
+        const typename E::vec2 v0 = E::cvt2(dv[db][4 * q4 + 0], dv[db][4 * q4 + 1]);
+        const typename E::vec2 v1 = E::cvt2(dv[db][4 * q4 + 2], dv[db][4 * q4 + 3]);
+        typename E::vec4 xk = {k0[0], k0[1], k1[0], k1[1]};
+        typename E::vec4 xv = {v0[0], v0[1], v1[0], v1[1]};
+        *reinterpret_cast<typename E::vec4*>(krow + 32 * db + 8 * q4 + 4 * g) = xk;
+        *reinterpret_cast<typename E::vec4*>(vrow + 32 * db + 8 * q4 + 4 * g) = xv;
+      }
+  }
+}
+
+template <typename Tag, int D, bool CAUSAL, bool DOC>
+static int launch_one(const KArgs& a, hipStream_t s) {
+  constexpr int BK = 128, BQ = 64;
+  const int nKt = (a.N + BK - 1) / BK;
+  const int slots = (a.B * a.H + 7) / 8;
+  const size_t lds = 4 * BQ * D * 2 + 2 * 768;
+  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(8 * slots * nKt), dim3(256), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <typename Tag, int D>
+static int launch_cd(const KArgs& a, bool causal, bool doc, hipStream_t s) {
+  if (causal) return doc ? launch_one<Tag, D, true, true>(a, s) : launch_one<Tag, D, true, false>(a, s);
+  return doc ? launch_one<Tag, D, false, true>(a, s) : launch_one<Tag, D, false, false>(a, s);
+}
+
+template <typename Tag>
+static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) {
+  switch (D) {
+    case 128: return launch_cd<Tag, 128>(a, causal, doc, s);
+    case 64: return launch_cd<Tag, 64>(a, causal, doc, s);
+    case 32: return launch_cd<Tag, 32>(a, causal, doc, s);
+    default: return -1;
+  }
+}
+
+int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s) {
+  return dtype == FA_DTYPE_BF16 ? launch_d<bf16_t>(a, D, causal, doc, s) : launch_d<fp16_t>(a, D, causal, doc, s);
+}
+
+}  // namespace fa

@@ -1,0 +1,212 @@
+// Shared device/host definitions for the gfx950 flash-attention kernels.
+//
+// Register-level conventions used by every compute kernel in this directory
+// (CDNA4 v_mfma_f32_32x32x16_{bf16,f16}, wave64):
+//   A operand (32 x 16): lane l holds row  (l & 31), k = 8*(l >> 5) .. +7
+//   B operand (16 x 32): lane l holds col  (l & 31), k = 8*(l >> 5) .. +7
+//   C/D       (32 x 32): lane l holds col  (l & 31), register r (0..15) is
+//                        row 8*(r >> 2) + 4*(l >> 5) + (r & 3)
+// ds_read_b64_tr_b16: inside each group of 16 lanes, result lane i, element e is
+// taken from source lane 4*e + (i >> 2), element (i & 3) of its 8-byte read.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/flash_mi355.h"
+
+namespace fa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+#define FA_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define FA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FA_DEV __device__ __forceinline__
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Rows covered by one entry of the id summaries written by the mask plan.
+constexpr int kSumRows = 64;
+
+struct bf16_t {};
+struct fp16_t {};
+
+template <typename Tag> struct Elem;
+
+template <> struct Elem<bf16_t> {
+  typedef __bf16 scalar;
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  typedef bf16x2 vec2;
+  static FA_DEV f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static FA_DEV vec4 lds_tr(const void* p) {
+    return __builtin_bit_cast(vec4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p)));
+  }
+  static FA_DEV vec2 cvt2(float x, float y) {
+    f32x2 t = {x, y};
+    return __builtin_convertvector(t, vec2);
+  }
+};
+
+template <> struct Elem<fp16_t> {
+  typedef _Float16 scalar;
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  typedef f16x2 vec2;
+  static FA_DEV f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static FA_DEV vec4 lds_tr(const void* p) {
+    return __builtin_bit_cast(vec4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p)));
+  }
+  static FA_DEV vec2 cvt2(float x, float y) {
+    f32x2 t = {x, y};
+    return __builtin_convertvector(t, vec2);
+  }
+};
+
+// Sign flip of 8 packed 16-bit floats (exact for both bf16 and fp16).
+template <typename E>
+FA_DEV typename E::vec8 neg8(typename E::vec8 x) {
+  i32x4 u = __builtin_bit_cast(i32x4, x);
+  u ^= (int)0x80008000;
+  return __builtin_bit_cast(typename E::vec8, u);
+}
+
+// Exchange between lane l and lane l ^ 32: returns the partner's value.
+FA_DEV float xhalf(float x) {
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // r[0] = {lo, lo}, r[1] = {hi, hi}: the partner of a low lane is r[1], of a high lane r[0]
+  unsigned lo = r[0], hi = r[1];
+  return __uint_as_float((threadIdx.x & 32) ? lo : hi);
+}
+FA_DEV float xhalf_max(float x) {
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+FA_DEV float xhalf_sum(float x) {
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+FA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+FA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---------------------------------------------------------------------------
+// Mask engine, element level.  keep(i, j) of the reference:
+//   tail   : j < N (and i < M at the store)             flash_triton.py:103-105
+//   causal : gap + i >= j, gap = max(0, N - M)          flash_triton.py:107
+//   doc    : eq_i >= 0 || eq_i == ek_j                  flash_triton.py:114
+// ---------------------------------------------------------------------------
+template <bool CAUSAL, bool DOC>
+FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j) {
+  bool keep = j < N;
+  if (CAUSAL) keep = keep && (gap + i >= j);
+  if (DOC) keep = keep && ((eq_i >= 0) || (eq_i == ek_j));
+  return keep;
+}
+
+// Summary of the ids of kSumRows consecutive rows (written by the mask plan).
+//   query side: lo/hi = min/max over rows with eq < 0 (lo > hi if none),
+//               glob  = 1 if any row has eq >= 0
+//   key side  : lo/hi = min/max over all keys of the tile
+struct IdSummary {
+  int lo, hi, glob, pad;
+};
+
+// A tile pair can hold a kept element only if a global query row exists or the
+// local-id interval of the query rows meets the id interval of the keys.
+FA_DEV bool doc_may_keep(int q_lo, int q_hi, int q_glob, int k_lo, int k_hi) {
+  return q_glob || (q_lo <= k_hi && k_lo <= q_hi);
+}
+// Every (row, key) pair of the tile pair passes the doc test.
+FA_DEV bool doc_all_keep(int q_lo, int q_hi, int k_lo, int k_hi) {
+  // no local row at all, or one local id shared by every key
+  return (q_lo > q_hi) || (q_lo == q_hi && k_lo == k_hi && q_lo == k_lo);
+}
+
+// Kernel-side view of the operands (built on the host from fa_params).
+struct KArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* delta;
+  const int* eq32;        // [B, Hq', Mp]
+  const int* ek32;        // [B, Hk', Np]
+  const IdSummary* qsum;  // [B, Hq', nQs]
+  const IdSummary* ksum;  // [B, Hk', nKs]
+  int64_t q_bs, q_hs, q_rs;
+  int64_t k_bs, k_hs, k_rs;
+  int64_t v_bs, v_hs, v_rs;
+  int64_t o_bs, o_hs, o_rs;
+  int64_t do_bs, do_hs, do_rs;
+  int64_t dq_bs, dq_hs, dq_rs;
+  int64_t dk_bs, dk_hs, dk_rs;
+  int64_t dv_bs, dv_hs, dv_rs;
+  int64_t eq_bs, eq_hs;   // strides of eq32 (head stride 0 when shared)
+  int64_t ek_bs, ek_hs;
+  int64_t qs_bs, qs_hs;   // strides of qsum in entries
+  int64_t ks_bs, ks_hs;
+  int B, H, Hk, G, M, N, gap;
+  int nQs, nKs;           // summary entries per (b, h)
+  float scale;            // sm_scale
+  float scale_log2e;      // sm_scale * log2(e)
+};
+
+// Workspace layout shared by host and device code.
+struct WsLayout {
+  int Hq1, Hk1;           // heads stored for eq / ek (1 when the head stride is 0)
+  int Mp, Np;             // M, N rounded up to kSumRows
+  int nQs, nKs;
+  uint64_t off_eq32, off_ek32, off_qsum, off_ksum, total;  // bytes
+};
+
+inline WsLayout ws_layout(const fa_params* p) {
+  WsLayout w;
+  w.Hq1 = (p->eq_stride[1] == 0) ? 1 : p->H;
+  w.Hk1 = (p->ek_stride[1] == 0) ? 1 : p->H;
+  w.nQs = (p->M + kSumRows - 1) / kSumRows;
+  w.nKs = (p->N + kSumRows - 1) / kSumRows;
+  w.Mp = w.nQs * kSumRows;
+  w.Np = w.nKs * kSumRows;
+  uint64_t o = 0;
+  auto take = [&](uint64_t bytes) { uint64_t r = o; o += (bytes + 255) & ~uint64_t(255); return r; };
+  w.off_eq32 = take(uint64_t(p->B) * w.Hq1 * w.Mp * 4);
+  w.off_ek32 = take(uint64_t(p->B) * w.Hk1 * w.Np * 4);
+  w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
+  w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
+  w.total = o;
+  return w;
+}
+
+// Launchers implemented one per translation unit; each returns a hipError_t as int.
+int launch_fwd(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+int launch_bwd_delta(const KArgs& a, int dtype, int D, hipStream_t s);
+int launch_bwd_dq(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s);
+int launch_mask_dump(const KArgs& a, bool causal, bool doc, uint8_t* out, hipStream_t s);
+
+}  // namespace fa

@@ -1,0 +1,12 @@
+"""MI355X (gfx950) flash attention with flexible masks.
+
+    from flash_mi355 import attention, SCORE_FUNC_MODE1_DOC
+    out = attention(q, k, v, causal=True, eq=eq, ek=ek, score_func_mode=SCORE_FUNC_MODE1_DOC)
+
+The four public names match the reference module ``flash_triton``.
+"""
+from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, FlashAttention, attention,
+                  attention_with_lse, mask_dump, maybe_contiguous)
+
+__all__ = ["attention", "FlashAttention", "SCORE_FUNC_MODE0_NOPE", "SCORE_FUNC_MODE1_DOC",
+           "attention_with_lse", "mask_dump", "maybe_contiguous"]

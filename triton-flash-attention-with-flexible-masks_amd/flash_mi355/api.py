@@ -1,0 +1,224 @@
+"""Drop-in operator: ``attention(q, k, v, causal, sm_scale, eq, ek, score_func_mode)``.
+
+Same entry point, argument order, defaults, checks and return values as the
+reference's ``flash_triton.attention`` / ``FlashAttention`` (flash_triton.py:506-641);
+the kernels behind it are the hand-written gfx950 kernels of libflash_mi355.so.
+torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _cabi
+
+SCORE_FUNC_MODE0_NOPE = 0  # flash_triton.py:20
+SCORE_FUNC_MODE1_DOC = 1   # flash_triton.py:22
+
+_DTYPES = {torch.bfloat16: _cabi.FA_DTYPE_BF16, torch.float16: _cabi.FA_DTYPE_FP16}
+_ID_DTYPES = {torch.int32: _cabi.FA_IDTYPE_I32, torch.int64: _cabi.FA_IDTYPE_I64}
+
+
+def maybe_contiguous(x):
+    """Innermost dimension must be contiguous (flash_triton.py:435-437)."""
+    return x.contiguous() if x.stride(-1) != 1 else x
+
+
+def _aligned(x):
+    """16-byte aligned base and outer strides that are multiples of 8 elements."""
+    ok = x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+    return x if ok else x.contiguous()
+
+
+def _set4(dst, t):
+    for i in range(4):
+        dst[i] = t.stride(i)
+
+
+def _set3(dst, t):
+    for i in range(3):
+        dst[i] = t.stride(i)
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class _Plan:
+    """fa_params filled in for one problem, plus the tensors that keep its pointers alive."""
+
+    def __init__(self, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+        B, H, M, D = q.shape
+        N, Hk = k.shape[2], k.shape[1]
+        p = _cabi.FaParams()
+        p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        _set4(p.q_stride, q); _set4(p.k_stride, k); _set4(p.v_stride, v)
+        p.B, p.H, p.Hk, p.M, p.N, p.D = B, H, Hk, M, N, D
+        p.causal = 1 if causal else 0
+        p.score_mode = int(score_func_mode)
+        p.dtype = _DTYPES[q.dtype]
+        p.sm_scale = float(sm_scale)
+        p.flags = 0
+        self.keep = [q, k, v]
+        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+            p.eq, p.ek = eq.data_ptr(), ek.data_ptr()
+            _set3(p.eq_stride, eq); _set3(p.ek_stride, ek)
+            p.id_dtype = _ID_DTYPES[eq.dtype]
+            self.keep += [eq, ek]
+        self.p = p
+        self.workspace = None
+
+    def ensure_workspace(self, device):
+        L = _cabi.lib()
+        nbytes = int(L.fa_workspace_bytes(ctypes.byref(self.p)))
+        if nbytes and self.workspace is None:
+            self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self.p.workspace = self.workspace.data_ptr()
+            self.p.workspace_bytes = nbytes
+            _cabi.check(L.fa_mask_plan(ctypes.byref(self.p), _stream_ptr(device)), "fa_mask_plan")
+
+
+def _prep_ids(e, name):
+    assert e.dim() == 3, f"{name} must be [bs, H, L]"
+    if e.dtype not in _ID_DTYPES:
+        assert not e.dtype.is_floating_point and e.dtype != torch.bool, f"{name} must be an integer tensor"
+        e = e.to(torch.int32) if e.dtype in (torch.int8, torch.int16, torch.uint8) else e.to(torch.int64)
+    return e
+
+
+class FlashAttention(torch.autograd.Function):
+    """Mirror of the reference autograd function (flash_triton.py:506-638)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+        # -- checks of flash_triton.py:510-530, same order and messages --
+        Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+        assert Dq == Dk and Dk == Dv, "feature size of q, k, v should be equal"
+        assert Dk in {16, 32, 64, 128}
+        B, H, M, D = q.shape
+        N = k.shape[2]
+        Hk, Hv = k.shape[1], v.shape[1]
+        assert Hk == Hv, "num of heads in k and v should be equal"
+        assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+        num_groups = H // Hk
+        assert (N >= M) or (not causal), "KV length should be larger than M length in causal mode!"
+        MN_GAP = max(0, N - M)
+        if sm_scale is None:
+            sm_scale = 1. / math.sqrt(D)
+        q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
+        assert (eq is None) == (ek is None)
+        if eq is None:
+            assert score_func_mode == SCORE_FUNC_MODE0_NOPE
+        # -- checks the reference leaves to the Triton launcher --
+        assert score_func_mode in (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC), "unknown score_func_mode"
+        assert q.is_cuda and k.is_cuda and v.is_cuda, "flash_mi355 runs on the GPU only"
+        assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, \
+            "q, k, v must share one of torch.bfloat16 / torch.float16"
+        assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
+        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+            eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
+            assert eq.dtype == ek.dtype or True
+            if eq.dtype != ek.dtype:
+                eq, ek = eq.to(torch.int64), ek.to(torch.int64)
+            assert tuple(eq.shape) == (B, H, M), "eq must be [bs, H, Lq]"
+            assert tuple(ek.shape) == (B, H, N), "ek must be [bs, H, Lk]"
+        else:
+            eq = ek = None
+        q, k, v = _aligned(q), _aligned(k), _aligned(v)
+
+        L = _cabi.lib()
+        with torch.cuda.device(q.device):
+            plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+            Out = torch.empty_like(q, memory_format=torch.contiguous_format)
+            lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
+            p = plan.p
+            p.o, p.lse = Out.data_ptr(), lse.data_ptr()
+            _set4(p.o_stride, Out)
+            plan.ensure_workspace(q.device)
+            _cabi.check(L.fa_fwd(ctypes.byref(p), _stream_ptr(q.device)), "fa_fwd")
+        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.workspace)
+        ctx.sm_scale = sm_scale
+        ctx.causal = causal
+        ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
+        ctx.score_func_info = (score_func_mode,)
+        return Out
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, lse, eq, ek, workspace = ctx.saved_tensors
+        B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
+        score_func_mode, = ctx.score_func_info
+        L = _cabi.lib()
+        do = _aligned(maybe_contiguous(do))
+        with torch.cuda.device(q.device):
+            plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode)
+            p = plan.p
+            if workspace is not None:   # the forward's mask plan is reused as is
+                plan.workspace = workspace
+                p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
+            delta = torch.empty_like(lse)
+            dq = torch.empty_like(q, memory_format=torch.contiguous_format)
+            dk = torch.empty((B, H, N, D), dtype=k.dtype, device=q.device)
+            dv = torch.empty((B, H, N, D), dtype=v.dtype, device=q.device)
+            p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+            p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+            _set4(p.o_stride, o); _set4(p.do_stride, do)
+            _set4(p.dq_stride, dq); _set4(p.dk_stride, dk); _set4(p.dv_stride, dv)
+            stream = _stream_ptr(q.device)
+            _cabi.check(L.fa_bwd_delta(ctypes.byref(p), stream), "fa_bwd_delta")
+            _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
+            _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
+            if num_groups > 1:  # flash_triton.py:635-637
+                dk = dk.reshape((B, Hk, num_groups, N, D)).sum(2, dtype=torch.float32).to(k.dtype)
+                dv = dv.reshape((B, Hk, num_groups, N, D)).sum(2, dtype=torch.float32).to(v.dtype)
+        return dq, dk, dv, None, None, None, None, None
+
+
+def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE):
+    """flash_triton.py:640-641."""
+    return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+
+
+# ---------------------------------------------------------------------------
+# Accessors for tests and benchmarks (not part of the reference's surface).
+# ---------------------------------------------------------------------------
+def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
+                       score_func_mode=SCORE_FUNC_MODE0_NOPE):
+    """Forward only; returns (O, LSE) with LSE in natural-log units (-inf for empty rows)."""
+    class _Ctx:
+        def save_for_backward(self, *t):
+            self.saved = t
+    ctx = _Ctx()
+    with torch.no_grad():
+        out = FlashAttention.forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+    return out, ctx.saved[4] * math.log(2.0)
+
+
+def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda"):
+    """keep(i, j) as a bool tensor [B, H, M, N], evaluated by the device mask routine."""
+    L = _cabi.lib()
+    device = torch.device(device)
+    p = _cabi.FaParams()
+    p.B, p.H, p.Hk, p.M, p.N, p.D = B, H, H, M, N, 64
+    p.causal = 1 if causal else 0
+    p.score_mode = int(score_func_mode)
+    p.dtype = _cabi.FA_DTYPE_BF16
+    keep = []
+    with torch.cuda.device(device):
+        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+            eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
+            if eq.dtype != ek.dtype:
+                eq, ek = eq.to(torch.int64), ek.to(torch.int64)
+            p.eq, p.ek = eq.data_ptr(), ek.data_ptr()
+            _set3(p.eq_stride, eq); _set3(p.ek_stride, ek)
+            p.id_dtype = _ID_DTYPES[eq.dtype]
+            nbytes = int(L.fa_workspace_bytes(ctypes.byref(p)))
+            ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+            keep += [eq, ek, ws]
+            _cabi.check(L.fa_mask_plan(ctypes.byref(p), _stream_ptr(device)), "fa_mask_plan")
+        out = torch.empty((B, H, M, N), dtype=torch.uint8, device=device)
+        _cabi.check(L.fa_mask_dump(ctypes.byref(p), out.data_ptr(), _stream_ptr(device)), "fa_mask_dump")
+    return out.bool()

@@ -1,0 +1,75 @@
+"""Build the gfx950 shared library in-tree with hipcc (cross-compiles without a GPU).
+
+    python -m flash_mi355.build          # from the package directory, or
+    flash_mi355.build.build(force=True)
+
+Every .hip file of csrc/ is compiled to an object next to the library and linked
+into flash_mi355/libflash_mi355.so.  Nothing is installed outside the tree.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR.parent / "csrc"
+INCLUDE = PKG_DIR.parent.parent / "include"
+LIB_PATH = PKG_DIR / "libflash_mi355.so"
+OBJ_DIR = PKG_DIR / "_obj"
+
+SOURCES = ["fa_api.hip", "fa_aux.hip", "fa_fwd.hip", "fa_bwd_dq.hip", "fa_bwd_dkdv.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # no compiler-generated packed fp32 arithmetic on this target
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(src: Path, obj: Path, extra) -> str:
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, f"-I{INCLUDE}", "-c", str(src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stderr[-4000:]}")
+    return r.stderr
+
+
+def build(force: bool = True, verbose: bool = False, extra_flags=()) -> Path:
+    """Compile all kernels and link the library; returns its path."""
+    OBJ_DIR.mkdir(exist_ok=True)
+    headers = list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h"))
+    newest_hdr = max(h.stat().st_mtime for h in headers)
+    jobs = []
+    for name in SOURCES:
+        src = CSRC / name
+        obj = OBJ_DIR / (src.stem + ".o")
+        stale = force or not obj.exists() or obj.stat().st_mtime < max(src.stat().st_mtime, newest_hdr)
+        if stale:
+            jobs.append((src, obj))
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        logs = list(ex.map(lambda j: _compile(j[0], j[1], list(extra_flags)), jobs))
+    if verbose:
+        for (src, _), log in zip(jobs, logs):
+            lines = [l for l in log.splitlines() if "packed-fp32-ops" not in l]
+            if lines:
+                print(f"--- {src.name}\n" + "\n".join(lines))
+    objs = [str(OBJ_DIR / (Path(n).stem + ".o")) for n in SOURCES]
+    if jobs or not LIB_PATH.exists():
+        cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *objs]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(force="--incremental" not in sys.argv, verbose=True)
+    print(path)

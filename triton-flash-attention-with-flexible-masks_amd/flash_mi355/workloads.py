@@ -1,0 +1,139 @@
+"""Seeded synthetic workloads for the benchmark and the parity tests, and the
+FLOP accounting used to report throughput.
+
+The five named configurations follow the benchmark definition of this project
+(document ids: negative = attend inside the own document only, >= 0 = attend to
+everything, the id semantics of the reference's sampler, testing.py:110-120).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+
+@dataclass
+class Workload:
+    name: str
+    B: int
+    H: int
+    Hk: int
+    Lq: int
+    Lk: int
+    D: int
+    dtype: str            # "bf16" | "fp16" | "fp32"
+    causal: bool
+    doc: bool
+    eq: Optional[np.ndarray] = None   # [B, Lq] int32 (shared by all heads)
+    ek: Optional[np.ndarray] = None   # [B, Lk] int32
+
+
+def _pack_docs(rng, L, draw_len):
+    """ids -(doc+1) for documents packed back to back until L tokens are covered."""
+    ids = np.empty(L, dtype=np.int32)
+    pos, doc = 0, 0
+    while pos < L:
+        n = int(draw_len(rng))
+        ids[pos:pos + n] = -(doc + 1)
+        pos += n
+        doc += 1
+    return ids
+
+
+def _globalise(rng, ids, frac):
+    ids = ids.copy()
+    ids[rng.random(ids.shape[0]) < frac] = 0
+    return ids
+
+
+def doc_ids_uniform(rng, L, lo, hi, global_frac):
+    return _globalise(rng, _pack_docs(rng, L, lambda r: r.integers(lo, hi + 1)), global_frac)
+
+
+def doc_ids_geometric(rng, L, mean, minimum, global_frac):
+    p = 1.0 / max(1.0, mean - minimum + 1)
+    return _globalise(rng, _pack_docs(rng, L, lambda r: minimum - 1 + r.geometric(p)), global_frac)
+
+
+def make_workload(name: str, seed: int = 0) -> Workload:
+    rng = np.random.default_rng(seed)
+    if name == "cfg1_cpu_doc_causal":
+        B, H, L, D = 2, 4, 512, 64
+        ids = np.stack([doc_ids_uniform(rng, L, 32, 256, 0.05) for _ in range(B)])
+        return Workload(name, B, H, H, L, L, D, "fp32", True, True, ids, ids)
+    if name == "cfg2_plain":
+        return Workload(name, 4, 16, 16, 2048, 2048, 64, "bf16", False, False)
+    if name == "cfg3_doc_causal_4k":
+        B, H, L, D = 2, 32, 4096, 128
+        ids = np.stack([doc_ids_uniform(rng, L, 128, 1024, 0.10) for _ in range(B)])
+        return Workload(name, B, H, H, L, L, D, "bf16", True, True, ids, ids)
+    if name == "cfg4_doc_causal_16k":
+        B, H, L, D = 1, 32, 16384, 128
+        ids = np.stack([doc_ids_geometric(rng, L, 512, 16, 0.02) for _ in range(B)])
+        return Workload(name, B, H, H, L, L, D, "bf16", True, True, ids, ids)
+    if name == "cfg5_rect_fp16":
+        B, H, Lq, Lk, D = 8, 8, 1024, 8192, 128
+        ek = np.repeat(-(np.arange(32, dtype=np.int32) + 1), Lk // 32)          # 32 docs of 256 keys
+        ek = np.broadcast_to(ek, (B, Lk)).copy()
+        eq = np.stack([_globalise(rng, ek[b, -Lq:], 0.05) for b in range(B)])   # the last 4 docs
+        return Workload(name, B, H, H, Lq, Lk, D, "fp16", True, True, eq, ek)
+    raise KeyError(name)
+
+
+WORKLOADS = ("cfg1_cpu_doc_causal", "cfg2_plain", "cfg3_doc_causal_4k", "cfg4_doc_causal_16k", "cfg5_rect_fp16")
+
+
+def keep_rows(w: Workload, b: int, i0: int, i1: int) -> np.ndarray:
+    """keep(i, j) for rows i0..i1 of batch b as a bool array [i1-i0, Lk]."""
+    i = np.arange(i0, i1, dtype=np.int64)[:, None]
+    j = np.arange(w.Lk, dtype=np.int64)[None, :]
+    keep = np.ones((i1 - i0, w.Lk), dtype=bool)
+    if w.causal:
+        keep &= (max(0, w.Lk - w.Lq) + i) >= j
+    if w.doc:
+        e_q = w.eq[b, i0:i1].astype(np.int64)[:, None]
+        e_k = w.ek[b].astype(np.int64)[None, :]
+        keep &= (e_q >= 0) | (e_q == e_k)
+    return keep
+
+
+def count_mask(w: Workload, tile: int = 128):
+    """(kept elements, non-empty canonical tile x tile tiles, all tiles) summed over the batch
+    (ids are shared by the heads, so per-head counts are these numbers)."""
+    kept = tiles = 0
+    n_tiles_k = (w.Lk + tile - 1) // tile
+    for b in range(w.B):
+        for i0 in range(0, w.Lq, tile):
+            k = keep_rows(w, b, i0, min(w.Lq, i0 + tile))
+            kept += int(k.sum())
+            col_any = k.any(axis=0)
+            pad = n_tiles_k * tile - w.Lk
+            if pad:
+                col_any = np.concatenate([col_any, np.zeros(pad, bool)])
+            tiles += int(col_any.reshape(n_tiles_k, tile).any(axis=1).sum())
+    total_tiles = w.B * ((w.Lq + tile - 1) // tile) * n_tiles_k
+    return kept, tiles, total_tiles
+
+
+def flops(w: Workload, mode: str = "fwd", kept=None, tiles=None, tile: int = 128):
+    """FLOP counts under the three conventions used in the reports.
+
+    dense : 4*B*H*Lq*Lk*D, halved when causal (testing.py:94-98; exact bottom-right
+            count for rectangular shapes)
+    elem  : 4*D*H*#kept elements
+    tile  : 4*D*H*tile^2*#canonical tiles with at least one kept element
+    backward = 2.5 x forward, forward+backward = 3.5 x (testing.py:103-105).
+    """
+    if kept is None or tiles is None:
+        kept, tiles, _ = count_mask(w, tile)
+    mult = {"fwd": 1.0, "bwd": 2.5, "fb": 3.5}[mode]
+    dense_pairs = w.Lq * w.Lk
+    if w.causal:
+        gap = max(0, w.Lk - w.Lq)
+        dense_pairs = w.Lq * gap + w.Lq * (w.Lq + 1) // 2 if w.Lq != w.Lk else w.Lq * w.Lk / 2
+    return {
+        "dense": 4.0 * w.B * w.H * dense_pairs * w.D * mult,
+        "elem": 4.0 * w.D * w.H * kept * mult,
+        "tile": 4.0 * w.D * w.H * tile * tile * tiles * mult,
+    }
