@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the flexible-mask attention operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+A step is one forward + backward pass of the drop-in operator
+(``attention(...)`` then ``.backward(dO)``) over one batch of the workload, with
+every input already resident in HBM.  Default workload: the headline
+configuration (bf16, causal + document mask, B=1 H=32 L=16384 D=128).
+
+One JSON line is printed.  ``value`` is forward+backward throughput in TFLOP/s
+under the tile-effective convention: 4*D*128*128 FLOPs for every canonical
+128x128 tile of the score matrix that holds at least one kept element, times 3.5
+for forward + backward (the reference's own accounting, testing.py:94-108, minus
+the tiles the mask empties).  Dense-equivalent and element-effective figures,
+forward and backward separately, are in ``detail``.
+
+``roofline`` is for the longest-running kernel of the step: algorithmic FLOPs of
+that kernel (tile-effective forward FLOPs x 1 for the forward, x 2 for dk/dv
+(4 GEMMs), x 1.5 for dq (3 GEMMs)) over its mean duration measured with HIP
+events on the launch stream, against the 2.5 PFLOP/s bf16 MFMA peak.
+``cpu_baseline`` times the reference's eager mask-materialising path on the host
+cores for a bounded sample (a few heads) of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "triton-flash-attention-with-flexible-masks_amd"))
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}   # MI355X dense MFMA peak
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); filled per (workload, kernel); None = not measured.
+MEASURED_TRAFFIC = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg4_doc_causal_16k")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-heads", type=int, default=2, help="(batch, head) slices timed on the CPU")
+    return ap.parse_args()
+
+
+def make_inputs(w, torch):
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[w.dtype]
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = torch.randn(w.B, w.H, w.Lq, w.D, device=dev, generator=g).to(dt)
+    k = torch.randn(w.B, w.Hk, w.Lk, w.D, device=dev, generator=g).to(dt)
+    v = torch.randn(w.B, w.Hk, w.Lk, w.D, device=dev, generator=g).to(dt)
+    do = torch.randn(w.B, w.H, w.Lq, w.D, device=dev, generator=g).to(dt)
+    eq = ek = None
+    if w.doc:  # ids shared by the heads, passed head-expanded as the reference harness does (testing.py:118)
+        eq = torch.from_numpy(w.eq).to(dev)[:, None, :].expand(w.B, w.H, w.Lq)
+        ek = torch.from_numpy(w.ek).to(dev)[:, None, :].expand(w.B, w.H, w.Lk)
+    return q, k, v, do, eq, ek
+
+
+def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
+    """Mean duration (ms) of every kernel of the step, each launched alone through the C ABI."""
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    L = _cabi.lib()
+    dev = q.device
+    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else 0)
+    p = plan.p
+    o = torch.empty_like(q)
+    lse = torch.empty(w.B, w.H, w.Lq, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    dq = torch.empty_like(q)
+    dk = torch.empty(w.B, w.H, w.Lk, w.D, device=dev, dtype=q.dtype)
+    dv = torch.empty_like(dk)
+    p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+        _set4(getattr(p, f), t)
+    plan.ensure_workspace(dev)
+    stream = _stream_ptr(dev)
+    ref = ctypes.byref(p)
+    out = {}
+    names = [("fa_fwd", L.fa_fwd), ("fa_bwd_delta", L.fa_bwd_delta), ("fa_bwd_dkdv", L.fa_bwd_dkdv), ("fa_bwd_dq", L.fa_bwd_dq)]
+    if w.doc:
+        names.insert(0, ("fa_mask_plan", L.fa_mask_plan))
+    for name, fn in names:
+        for _ in range(3):
+            _cabi.check(fn(ref, stream), name)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn(ref, stream)
+        e1.record()
+        e1.synchronize()
+        out[name] = e0.elapsed_time(e1) / iters
+    return out
+
+
+def cpu_baseline(w, heads, torch):
+    """The reference's eager path (testing.py:32-47) on the host cores for `heads` (b, h) slices."""
+    from oracle import attention_oracle as O
+    from flash_mi355 import workloads as W
+    cores = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+    n = min(heads, w.B * w.H)
+    t_total = 0.0
+    for s in range(n):
+        b = s % w.B
+        q = torch.randn(1, 1, w.Lq, w.D, generator=g).requires_grad_(True)
+        k = torch.randn(1, 1, w.Lk, w.D, generator=g).requires_grad_(True)
+        v = torch.randn(1, 1, w.Lk, w.D, generator=g).requires_grad_(True)
+        do = torch.randn(1, 1, w.Lq, w.D, generator=g)
+        keep = None
+        if w.doc:
+            e_q = torch.from_numpy(w.eq[b])[:, None]
+            e_k = torch.from_numpy(w.ek[b])[None, :]
+            keep = ((e_q >= 0) | (e_q == e_k))[None, None]
+        t0 = time.perf_counter()
+        out = O.eager_attention_cpu(q, k, v, w.causal, keep)
+        out.backward(do)
+        t_total += time.perf_counter() - t0
+        del out, q, k, v, keep
+    per_slice = t_total / n
+    # dense-equivalent FLOPs with the x2.0 backward factor the reference applies to eager paths (testing.py:103)
+    f = W.flops(w, "fwd", kept=0, tiles=0)["dense"] / (w.B * w.H)
+    return {
+        "value": round(3.0 * f / per_slice * 1e-12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"{n} of {w.B * w.H} (batch, head) slices of {w.name}, fp32 eager fwd+bwd, "
+                  f"{per_slice:.2f} s per slice (dense-equivalent FLOPs, backward x2.0)",
+        "seconds_per_slice": round(per_slice, 3),
+        "extrapolated_step_seconds": round(per_slice * w.B * w.H, 1),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this operator shards over (batch, head) with no "
+              "communication and this build uses a single GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from flash_mi355 import attention, workloads as W
+
+    w = W.make_workload(args.workload)
+    q, k, v, do, eq, ek = make_inputs(w, torch)
+    mode = 1 if w.doc else 0
+    scale = 1.0 / math.sqrt(w.D)
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = attention(q, k, v, w.causal, scale, eq, ek, mode)
+        out.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    kept, tiles, total_tiles = W.count_mask(w)
+    f_fwd = W.flops(w, "fwd", kept, tiles)
+    kt = time_kernels(w, q.detach(), k.detach(), v.detach(), do, eq, ek, torch)
+    t_fwd = kt["fa_fwd"] + kt.get("fa_mask_plan", 0.0)
+    t_bwd = kt["fa_bwd_delta"] + kt["fa_bwd_dkdv"] + kt["fa_bwd_dq"]
+    peak = PEAK_TFLOPS[w.dtype]
+
+    def tf(flops, ms):
+        return flops / ms * 1e-9
+
+    detail = {"ms": {n: round(t, 4) for n, t in kt.items()},
+              "tiles_nonempty": tiles, "tiles_total": total_tiles,
+              "kept_fraction": round(kept / (w.B * w.Lq * w.Lk), 5)}
+    for conv in ("tile", "dense", "elem"):
+        detail[f"fwd_tflops_{conv}"] = round(tf(f_fwd[conv], t_fwd), 1)
+        detail[f"bwd_tflops_{conv}"] = round(tf(2.5 * f_fwd[conv], t_bwd), 1)
+    detail["fwd_pct_peak_tile"] = round(100 * detail["fwd_tflops_tile"] / peak, 2)
+    detail["bwd_pct_peak_tile"] = round(100 * detail["bwd_tflops_tile"] / peak, 2)
+
+    # roofline of the longest kernel: GEMMs that kernel executes, in tile-effective forward units
+    gemm_units = {"fa_fwd": 1.0, "fa_bwd_dkdv": 2.0, "fa_bwd_dq": 1.5}
+    dom = max(gemm_units, key=lambda n: kt[n])
+    achieved = tf(gemm_units[dom] * f_fwd["tile"], kt[dom])
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((w.name, dom)),
+                "avg_launch_ms": round(kt[dom], 4),
+                "all": {n: {"achieved": round(tf(u * f_fwd["tile"], kt[n]), 1),
+                            "frac": round(tf(u * f_fwd["tile"], kt[n]) / peak, 4)} for n, u in gemm_units.items()}}
+
+    value = tf(3.5 * f_fwd["tile"], ms_per_step)
+    line = {
+        "metric": "attention fwd+bwd TFLOP/s (bf16, doc+causal mask, tile-effective FLOPs)",
+        "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": w.name, "B": w.B, "H": w.H, "Hk": w.Hk, "Lq": w.Lq, "Lk": w.Lk, "D": w.D,
+                   "causal": w.causal, "doc_mask": w.doc},
+        "pct_of_mfma_peak": round(100 * value / peak, 2),
+        "detail": detail, "roofline": roofline,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(w, args.cpu_heads, torch)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
