@@ -93,21 +93,26 @@ static KArgs make_args(const fa_params* p) {
   a.gap = p->N > p->M ? p->N - p->M : 0;  // flash_triton.py:521
   a.scale = p->sm_scale;
   a.scale_log2e = p->sm_scale * kLog2e;
-  a.eq32 = nullptr; a.ek32 = nullptr; a.qsum = nullptr; a.ksum = nullptr;
-  a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
-  a.nQs = a.nKs = 0;
+  a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;
+  a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.pm_bs = a.pm_hs = a.qh_bs = a.qh_hs = 0;
+  a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
+  a.nQs = a.nKs = a.Pp = 0;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     const WsLayout w = ws_layout(p);
     char* ws = reinterpret_cast<char*>(p->workspace);
     a.eq32 = reinterpret_cast<const int*>(ws + w.off_eq32);
     a.ek32 = reinterpret_cast<const int*>(ws + w.off_ek32);
+    a.perm = reinterpret_cast<const int*>(ws + w.off_perm);
+    a.qhdr = reinterpret_cast<const QHeader*>(ws + w.off_qhdr);
     a.qsum = reinterpret_cast<const IdSummary*>(ws + w.off_qsum);
     a.ksum = reinterpret_cast<const IdSummary*>(ws + w.off_ksum);
     a.eq_bs = int64_t(w.Hq1) * w.Mp; a.eq_hs = w.Hq1 == 1 ? 0 : w.Mp;
     a.ek_bs = int64_t(w.Hk1) * w.Np; a.ek_hs = w.Hk1 == 1 ? 0 : w.Np;
+    a.pm_bs = int64_t(w.Hq1) * w.Pp; a.pm_hs = w.Hq1 == 1 ? 0 : w.Pp;
+    a.qh_bs = w.Hq1; a.qh_hs = w.Hq1 == 1 ? 0 : 1;
     a.qs_bs = int64_t(w.Hq1) * w.nQs; a.qs_hs = w.Hq1 == 1 ? 0 : w.nQs;
     a.ks_bs = int64_t(w.Hk1) * w.nKs; a.ks_hs = w.Hk1 == 1 ? 0 : w.nKs;
-    a.nQs = w.nQs; a.nKs = w.nKs;
+    a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
   }
   return a;
 }

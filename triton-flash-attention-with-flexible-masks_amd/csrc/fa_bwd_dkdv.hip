@@ -1,6 +1,6 @@
 // dK/dV kernel of the split backward: 128 keys per workgroup (32 per wave) held
-// in registers, query-side tiles (Q, dO, LSE, delta, eq) streamed through LDS.
-// Replaces _bwd_kv_kernel of the reference (flash_triton.py:175-321).
+// in registers, query-side tiles (Q, dO, LSE, delta, eq, row index) streamed
+// through LDS.  Replaces _bwd_kv_kernel of the reference (flash_triton.py:175-321).
 //
 //   S    = Q K^T           A = Q rows (LDS),  B = K^T (registers, whole kernel)
 //   dP   = dO V^T          A = dO rows (LDS), B = V^T (registers, whole kernel)
@@ -10,9 +10,15 @@
 //   dK^T += Q^T dS         A = Q^T  via ds_read_b64_tr_b16, B = dS
 //   dK   = dK * sm_scale                                 (flash_triton.py:313)
 // In the accumulator layout each lane owns ONE key column and 16 query rows of
-// every 32-row block, so LSE / delta / eq are read as broadcast 16-byte LDS loads.
+// every 32-row block, so LSE / delta / eq / row index are read as broadcast
+// 16-byte LDS loads.
+// With document ids the query side is walked in the permuted (local rows first)
+// order of the mask plan: tiles are gathered row by row through the permutation,
+// and only tiles whose id interval and row range can meet this workgroup's keys
+// are visited.
 // dK, dV are written per query head; the group sum for grouped-query attention is
 // done by the caller (flash_triton.py:635-637).
+
 #include "fa_tile.h"
 
 namespace fa {
@@ -25,18 +31,17 @@ void bwd_dkdv_kernel(const KArgs a) {
   using vec8 = typename E::vec8;
   constexpr int BK = 128, BQ = 64, KS = D / 16, DBN = D / 32;
   constexpr int TILE_BYTES = BQ * D * 2;
-  constexpr int AUX_OFF = 4 * TILE_BYTES;  // [2 buffers][3 arrays][64] x 4 bytes
+  constexpr int AUX_OFF = 4 * TILE_BYTES;  // [2 buffers][4 arrays][64] x 4 bytes
+  constexpr int AUX_BYTES = 1024;
+  using Loader = TileLoader<D, BQ>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lq = lane & 31, g = lane >> 5;
 
   const int nKt = (a.N + BK - 1) / BK;
-  const int BH = a.B * a.H;
-  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int bh = (idx / nKt) * 8 + xcd;
-  if (bh >= BH) return;
-  const int kt = idx % nKt;  // causal: the first key tiles see the most query rows
+  int kt, bh;
+  if (!block_to_tile(nKt, a.B * a.H, kt, bh)) return;  // causal: the first key tiles see the most rows
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
 
   const T* qp = reinterpret_cast<const T*>(a.q) + b * a.q_bs + h * a.q_hs;
@@ -66,10 +71,14 @@ void bwd_dkdv_kernel(const KArgs a) {
   int wk_lo = 0, wk_hi = 0;   // id interval of this wave's 32 keys
   int gk_lo = 0, gk_hi = 0;   // of the workgroup's 128 keys
   const int* eqp = nullptr;
+  const int* pmp = nullptr;
   const IdSummary* qsum = nullptr;
+  int nQtiles = (a.M + BQ - 1) / BQ;
+  int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
   if (DOC) {
     ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
     eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
+    pmp = a.perm + b * a.pm_bs + h * a.pm_hs;
     qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
     const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
     const IdSummary s0 = ks[n0 / kSumRows];
@@ -86,12 +95,24 @@ void bwd_dkdv_kernel(const KArgs a) {
       hi = max(hi, __shfl_xor(hi, off));
     }
     wk_lo = lo; wk_hi = hi;
+    nQtiles = a.nQs;
+    first = 0;
   }
-
-  const int nQtiles = (a.M + BQ - 1) / BQ;
-  const int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
   TileIter it;
-  it.init(first, nQtiles, qsum, gk_lo, gk_hi, 0, false);
+  it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000);
+
+  Loader ldQ, ldO;
+  ldQ.init(qp, a.q_rs, a.M);
+  ldO.init(dop, a.do_rs, a.M);
+  LdsOffsets<D> lo;
+  lo.init();
+  // gathered loads: byte offset of the lane's chunk inside its row, and the tile rows it fetches
+  int g_coff[Loader::PER], g_rit[Loader::PER];
+#pragma unroll
+  for (int i = 0; i < Loader::PER; ++i) {
+    g_rit[i] = (i * 4 + wave) * Loader::RPI + lane / Loader::CPR;
+    g_coff[i] = ((lane % Loader::CPR) ^ swz<D, SWZ_ROW>(g_rit[i])) * 16;
+  }
 
   f32x16 dk[DBN], dv[DBN];
 #pragma unroll
@@ -99,99 +120,144 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
+  // row indices of a permuted tile this lane needs: PER tile rows for Q/dO, one for the aux arrays
+  int ri_t[Loader::PER] = {};
+  int ri_aux = 0;
+  auto fetch_idx = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < Loader::PER; ++i) ri_t[i] = pmp[tile * BQ + g_rit[i]];
+    ri_aux = pmp[tile * BQ + lane];
+  };
   auto load_tile = [&](int tile, int bufi) {
-    const int m0 = tile * BQ;
-    tile_load_async<T, D, BQ, SWZ_ROW>(qp, a.q_rs, m0, a.M, smem + bufi * TILE_BYTES);
-    tile_load_async<T, D, BQ, SWZ_ROW>(dop, a.do_rs, m0, a.M, smem + (2 + bufi) * TILE_BYTES);
-    const int r = m0 + lane < a.M ? m0 + lane : a.M - 1;
-    char* aux = smem + AUX_OFF + bufi * 768;
-    if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
-    if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
-    if (DOC && wave == 2) __builtin_amdgcn_global_load_lds(FA_GLB(eqp + r), FA_LDS(aux + 512), 4, 0, 0);
+    char* aux = smem + AUX_OFF + bufi * AUX_BYTES;
+    if (!DOC) {
+      const int m0 = tile * BQ;
+      ldQ.issue(m0, smem + bufi * TILE_BYTES);
+      ldO.issue(m0, smem + (2 + bufi) * TILE_BYTES);
+      const int r = m0 + lane < a.M ? m0 + lane : a.M - 1;
+      if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
+      if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < Loader::PER; ++i) {
+        const int r = ri_t[i] >= 0 ? ri_t[i] : 0;
+        buf_load_lds16(ldQ.rsrc, smem + bufi * TILE_BYTES + (i * 4 + wave) * 1024, r * ldQ.row_bytes + g_coff[i], 0);
+        buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * 4 + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
+      }
+      const int r = ri_aux >= 0 ? ri_aux : 0;
+      if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
+      if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
+      if (wave == 2) __builtin_amdgcn_global_load_lds(FA_GLB(eqp + r), FA_LDS(aux + 512), 4, 0, 0);
+      if (wave == 3) __builtin_amdgcn_global_load_lds(FA_GLB(pmp + tile * BQ + lane), FA_LDS(aux + 768), 4, 0, 0);
+    }
   };
 
-  int cur = it.next();
-  int buf = 0;
-  if (cur >= 0) load_tile(cur, 0);
-  while (cur >= 0) {
-    const int nxt = it.next();
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) load_tile(nxt, buf ^ 1);
-    const char* lqt = smem + buf * TILE_BYTES;
-    const char* ldo = smem + (2 + buf) * TILE_BYTES;
-    const char* aux = smem + AUX_OFF + buf * 768;
-    const int m0 = cur * BQ;
+  auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
+    const char* lqt = smem + BUF * TILE_BYTES;
+    const char* ldo = smem + (2 + BUF) * TILE_BYTES;
+    const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
+    const int m0 = cur * BQ;  // natural order only
 
-    // wave-level decisions: rows m0..m0+63 against keys nw..nw+31
-    bool skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
-    bool need_mask = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
-    if (DOC) {
+    // wave-level decisions: the tile's 64 rows against keys nw..nw+31
+    bool skip, need_mask;
+    if (!DOC) {
+      skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
+      need_mask = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
+    } else {
       const IdSummary qs = qsum[cur];
-      skip = skip || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
-      need_mask = need_mask || !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
+      skip = (nw >= a.N) || (CAUSAL && (a.gap + qs.rmax < nw)) || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
+      need_mask = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31)) ||
+                  !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
     }
-    if (!skip) {
+    if (skip) return;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        f32x16 s, dp;
+    for (int qb = 0; qb < 2; ++qb) {
+      f32x16 s = zero, dp = zero;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 qa = lds_row8<E>(lqt + lo.row[ks] + qb * 32 * D * 2);
+        s = E::mfma32(qa, kf[ks], s);
+      }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 qa = frag_row<E, D, SWZ_ROW>(lqt, qb * 32 + lq, 2 * ks + g);
-          s = E::mfma32(qa, kf[ks], s);
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 da = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * D * 2);
+        dp = E::mfma32(da, vf[ks], dp);
+      }
+      // s -> P, dp -> dS for this lane's 16 query rows of the block
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
+        const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+        i32x4 eqv = {0, 0, 0, 0};
+        i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
+        if (DOC && need_mask) {
+          eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+          rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
         }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 da = frag_row<E, D, SWZ_ROW>(ldo, qb * 32 + lq, 2 * ks + g);
-          dp = E::mfma32(da, vf[ks], dp);
+        for (int t = 0; t < 4; ++t) {
+          float p = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
+          if (need_mask) {
+            const int i = rowv[t];
+            const bool keep = (i >= 0) && (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
+            p = keep ? p : 0.f;
+          }
+          s[4 * q4 + t] = p;
+          dp[4 * q4 + t] = p * (dp[4 * q4 + t] - dl[t]);
         }
-        // s -> P, dp -> dS for this lane's 16 query rows of the block
+      }
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
-          const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
-          const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
-          i32x4 eqv = {0, 0, 0, 0};
-          if (DOC && need_mask) eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+      for (int half = 0; half < 2; ++half) {
+        vec8 pf, dsf;
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            float p = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
-            if (need_mask) {
-              const int i = m0 + i0 + t;
-              const bool keep = (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
-              p = keep ? p : 0.f;
-            }
-            s[4 * q4 + t] = p;
-            dp[4 * q4 + t] = p * (dp[4 * q4 + t] - dl[t]);
-          }
+        for (int t = 0; t < 8; t += 2) {
+          const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
+          const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
+          pf[t] = pr[0]; pf[t + 1] = pr[1];
+          dsf[t] = dr[0]; dsf[t + 1] = dr[1];
+        }
+        const int goff = (2 * qb + half) * 16 * D * 2;
+#pragma unroll
+        for (int db = 0; db < DBN; ++db) {
+          const vec8 dot = lds_tr8<E>(ldo + lo.tr[db][0] + goff, ldo + lo.tr[db][1] + goff);
+          dv[db] = E::mfma32(dot, pf, dv[db]);
         }
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          vec8 pf, dsf;
-#pragma unroll
-          for (int t = 0; t < 8; t += 2) {
-            const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
-            const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
-            pf[t] = pr[0]; pf[t + 1] = pr[1];
-            dsf[t] = dr[0]; dsf[t + 1] = dr[1];
-          }
-#pragma unroll
-          for (int db = 0; db < DBN; ++db) {
-            const vec8 dot = frag_tr<E, D, SWZ_TR>(ldo, 32 * qb + 16 * half, db);
-            dv[db] = E::mfma32(dot, pf, dv[db]);
-          }
-#pragma unroll
-          for (int db = 0; db < DBN; ++db) {
-            const vec8 qtf = frag_tr<E, D, SWZ_TR>(lqt, 32 * qb + 16 * half, db);
-            dk[db] = E::mfma32(qtf, dsf, dk[db]);
-          }
+        for (int db = 0; db < DBN; ++db) {
+          const vec8 qtf = lds_tr8<E>(lqt + lo.tr[db][0] + goff, lqt + lo.tr[db][1] + goff);
+          dk[db] = E::mfma32(qtf, dsf, dk[db]);
         }
       }
     }
-    cur = nxt;
-    buf ^= 1;
+  };
+
+  // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and
+  // the row indices of the tile after that are fetched
+  int cur = it.next();
+  int nxt = cur >= 0 ? it.next() : -1;
+  if (cur >= 0) {
+    if (DOC) fetch_idx(cur);
+    load_tile(cur, 0);
+    if (DOC && nxt >= 0) fetch_idx(nxt);
+  }
+  while (cur >= 0) {
+    int nxt2 = nxt >= 0 ? it.next() : -1;
+    wait_async_loads();
+    __syncthreads();
+    if (nxt >= 0) load_tile(nxt, 1);
+    if (DOC && nxt2 >= 0) fetch_idx(nxt2);
+    compute(0, cur);
+    cur = nxt; nxt = nxt2;
+    if (cur < 0) break;
+    nxt2 = nxt >= 0 ? it.next() : -1;
+    wait_async_loads();
+    __syncthreads();
+    if (nxt >= 0) load_tile(nxt, 0);
+    if (DOC && nxt2 >= 0) fetch_idx(nxt2);
+    compute(1, cur);
+    cur = nxt; nxt = nxt2;
   }
 
   if (key < a.N) {
@@ -214,12 +280,13 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
 }
 
+
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BK = 128, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
   const int slots = (a.B * a.H + 7) / 8;
-  const size_t lds = 4 * BQ * D * 2 + 2 * 768;
+  const size_t lds = 4 * BQ * D * 2 + 2 * 1024;
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {

@@ -8,6 +8,7 @@
 //   dQ^T += K^T dS^T      A = K^T via ds_read_b64_tr_b16, B = dS^T from the accumulators
 //   dQ   = dQ * sm_scale                                  (flash_triton.py:425)
 // Same workgroup shape, LDS staging and tile skipping as the forward kernel.
+
 #include "fa_tile.h"
 
 namespace fa {
@@ -22,16 +23,17 @@ void bwd_dq_kernel(const KArgs a) {
   constexpr int TILE_BYTES = BN * D * 2;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int lq = lane & 31, g = lane >> 5;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 5;
 
-  const int nQt = (a.M + BM - 1) / BM;
-  const int BH = a.B * a.H;
-  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int bh = (idx / nQt) * 8 + xcd;
-  if (bh >= BH) return;
-  const int qt = nQt - 1 - (idx % nQt);
+  const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
+  int slot, bh;
+  if (!block_to_tile(nQt, a.B * a.H, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  QTileCtx<CAUSAL, DOC> qc;
+  if (!qc.init(a, b, h, nQt - 1 - slot)) return;
+  const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
+  const int* ekp = qc.ekp;
 
   const T* qp = reinterpret_cast<const T*>(a.q) + b * a.q_bs + h * a.q_hs;
   const T* kp = reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs;
@@ -40,11 +42,6 @@ void bwd_dq_kernel(const KArgs a) {
   T* dqp = reinterpret_cast<T*>(a.dq) + b * a.dq_bs + h * a.dq_hs;
   const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
   const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
-
-  const int m0 = qt * BM;
-  const int mw = m0 + wave * 32;
-  const int row = mw + lq;
-  const int rowc = row < a.M ? row : a.M - 1;
 
   vec8 qf[KS], dof[KS];
 #pragma unroll
@@ -57,36 +54,14 @@ void bwd_dq_kernel(const KArgs a) {
   if (L_i == -INFINITY) L_i = INFINITY;  // row without any kept key: P = exp2(-inf) = 0
   const float delta_i = delp[rowc];
 
-  int eq_i = 0;
-  int wq_lo = 0, wq_hi = -1, wq_glob = 1;
-  int gq_lo = 0, gq_hi = -1, gq_glob = 1;
-  const int* ekp = nullptr;
-  const IdSummary* ksum = nullptr;
-  if (DOC) {
-    eq_i = a.eq32[b * a.eq_bs + h * a.eq_hs + rowc];
-    ekp = a.ek32 + b * a.ek_bs + h * a.ek_hs;
-    ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
-    const IdSummary* qs = a.qsum + b * a.qs_bs + h * a.qs_hs;
-    const IdSummary s0 = qs[m0 / kSumRows];
-    gq_lo = s0.lo; gq_hi = s0.hi; gq_glob = s0.glob;
-    if (m0 / kSumRows + 1 < a.nQs) {
-      const IdSummary s1 = qs[m0 / kSumRows + 1];
-      gq_lo = min(gq_lo, s1.lo); gq_hi = max(gq_hi, s1.hi); gq_glob |= s1.glob;
-    }
-    const bool local = (eq_i < 0) && (row < a.M);
-    int lo = local ? eq_i : 0x7fffffff, hi = local ? eq_i : (int)0x80000000;
-#pragma unroll
-    for (int off = 16; off >= 1; off >>= 1) {
-      lo = min(lo, __shfl_xor(lo, off));
-      hi = max(hi, __shfl_xor(hi, off));
-    }
-    wq_lo = lo; wq_hi = hi;
-    wq_glob = __builtin_amdgcn_ballot_w64(eq_i >= 0 && row < a.M) != 0;
-  }
-
-  const int hi_key = CAUSAL ? min(a.N, a.gap + m0 + BM) : a.N;
   TileIter it;
-  it.init(0, (hi_key + BN - 1) / BN, ksum, gq_lo, gq_hi, gq_glob, true);
+  it.init_keys(0, (qc.hi_key(a) + BN - 1) / BN, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+
+  TileLoader<D, BN> ldK, ldV;
+  ldK.init(kp, a.k_rs, a.N);
+  ldV.init(vp, a.v_rs, a.N);
+  LdsOffsets<D> lo;
+  lo.init();
 
   f32x16 dq[DBN];
 #pragma unroll
@@ -94,88 +69,93 @@ void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-  int cur = it.next();
-  int buf = 0;
-  if (cur >= 0) {
-    tile_load_async<T, D, BN, SWZ_ROW>(kp, a.k_rs, cur * BN, a.N, smem + 0 * TILE_BYTES);
-    tile_load_async<T, D, BN, SWZ_ROW>(vp, a.v_rs, cur * BN, a.N, smem + 2 * TILE_BYTES);
-  }
-  while (cur >= 0) {
-    const int nxt = it.next();
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) {
-      tile_load_async<T, D, BN, SWZ_ROW>(kp, a.k_rs, nxt * BN, a.N, smem + (buf ^ 1) * TILE_BYTES);
-      tile_load_async<T, D, BN, SWZ_ROW>(vp, a.v_rs, nxt * BN, a.N, smem + (2 + (buf ^ 1)) * TILE_BYTES);
-    }
-    const char* lk = smem + buf * TILE_BYTES;
-    const char* lv = smem + (2 + buf) * TILE_BYTES;
+  auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
+    const char* lk = smem + BUF * TILE_BYTES;
+    const char* lv = smem + (2 + BUF) * TILE_BYTES;
     const int n0 = cur * BN;
-
-    bool skip = CAUSAL && (n0 > a.gap + mw + 31);
-    bool need_mask = (n0 + BN > a.N) || (CAUSAL && (n0 + BN - 1 > a.gap + mw));
-    if (DOC) {
-      const IdSummary ks = ksum[cur];
-      skip = skip || !doc_may_keep(wq_lo, wq_hi, wq_glob, ks.lo, ks.hi);
-      need_mask = need_mask || !doc_all_keep(wq_lo, wq_hi, ks.lo, ks.hi);
-    }
-    if (!skip) {
+    bool skip, need_mask;
+    qc.decide(a, cur, n0, BN, skip, need_mask);
+    if (skip) return;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        f32x16 s, dp;
+    for (int kb = 0; kb < 2; ++kb) {
+      f32x16 s = zero, dp = zero;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * D * 2);
+        s = E::mfma32(kf, qf[ks], s);
+      }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 kf = frag_row<E, D, SWZ_ROW>(lk, kb * 32 + lq, 2 * ks + g);
-          s = E::mfma32(kf, qf[ks], s);
-        }
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 vf = lds_row8<E>(lv + lo.row[ks] + kb * 32 * D * 2);
+        dp = E::mfma32(vf, dof[ks], dp);
+      }
+      // P and dS for this lane's 16 keys of the block
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 vf = frag_row<E, D, SWZ_ROW>(lv, kb * 32 + lq, 2 * ks + g);
-          dp = E::mfma32(vf, dof[ks], dp);
-        }
-        // P and dS for this lane's 16 keys of the block
+      for (int r = 0; r < 16; ++r) {
+        const float p = fast_exp2(__builtin_fmaf(s[r], c, -L_i));
+        s[r] = p * (dp[r] - delta_i);
+      }
+      if (need_mask) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float p = fast_exp2(__builtin_fmaf(s[r], c, -L_i));
-          s[r] = p * (dp[r] - delta_i);
-        }
-        if (need_mask) {
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int j0 = n0 + 32 * kb + 8 * q4 + 4 * g;
+          i32x4 ekv = {0, 0, 0, 0};
+          if (DOC) ekv = *reinterpret_cast<const i32x4*>(ekp + j0);
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const int j0 = n0 + 32 * kb + 8 * q4 + 4 * g;
-            i32x4 ekv = {0, 0, 0, 0};
-            if (DOC) ekv = *reinterpret_cast<const i32x4*>(ekp + j0);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              const bool keep = keep_elem<CAUSAL, DOC>(row, j0 + t, a.gap, a.N, eq_i, ekv[t]);
-              s[4 * q4 + t] = keep ? s[4 * q4 + t] : 0.f;
-            }
-          }
-        }
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          vec8 dsf;
-#pragma unroll
-          for (int t = 0; t < 8; t += 2) {
-            const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
-            dsf[t] = pr[0];
-            dsf[t + 1] = pr[1];
-          }
-#pragma unroll
-          for (int db = 0; db < DBN; ++db) {
-            const vec8 ktf = frag_tr<E, D, SWZ_TR>(lk, 32 * kb + 16 * half, db);
-            dq[db] = E::mfma32(ktf, dsf, dq[db]);
+          for (int t = 0; t < 4; ++t) {
+            const bool keep = keep_elem<CAUSAL, DOC>(row, j0 + t, a.gap, a.N, eq_i, ekv[t]);
+            s[4 * q4 + t] = keep ? s[4 * q4 + t] : 0.f;
           }
         }
       }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        vec8 dsf;
+#pragma unroll
+        for (int t = 0; t < 8; t += 2) {
+          const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
+          dsf[t] = pr[0];
+          dsf[t + 1] = pr[1];
+        }
+#pragma unroll
+        for (int db = 0; db < DBN; ++db) {
+          const int goff = (2 * kb + half) * 16 * D * 2;
+          const vec8 ktf = lds_tr8<E>(lk + lo.tr[db][0] + goff, lk + lo.tr[db][1] + goff);
+          dq[db] = E::mfma32(ktf, dsf, dq[db]);
+        }
+      }
     }
+  };
+
+  int cur = it.next();
+  if (cur >= 0) {
+    ldK.issue(cur * BN, smem + 0 * TILE_BYTES);
+    ldV.issue(cur * BN, smem + 2 * TILE_BYTES);
+  }
+  while (cur >= 0) {
+    int nxt = it.next();
+    wait_async_loads();
+    __syncthreads();
+    if (nxt >= 0) {
+      ldK.issue(nxt * BN, smem + 1 * TILE_BYTES);
+      ldV.issue(nxt * BN, smem + 3 * TILE_BYTES);
+    }
+    compute(0, cur);
     cur = nxt;
-    buf ^= 1;
+    if (cur < 0) break;
+    nxt = it.next();
+    wait_async_loads();
+    __syncthreads();
+    if (nxt >= 0) {
+      ldK.issue(nxt * BN, smem + 0 * TILE_BYTES);
+      ldV.issue(nxt * BN, smem + 2 * TILE_BYTES);
+    }
+    compute(1, cur);
+    cur = nxt;
   }
 
-  if (row < a.M) {
+  if (row >= 0) {
     T* drow = dqp + int64_t(row) * a.dq_rs;
     const float sc = a.scale;
 #pragma unroll
@@ -190,10 +170,11 @@ void bwd_dq_kernel(const KArgs a) {
   }
 }
 
+
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
-  const int nQt = (a.M + BM - 1) / BM;
+  const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
   const int slots = (a.B * a.H + 7) / 8;
   const size_t lds = 4 * BN * D * 2;
   auto kern = bwd_dq_kernel<Tag, D, CAUSAL, DOC>;

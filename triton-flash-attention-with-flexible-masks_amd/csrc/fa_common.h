@@ -122,12 +122,27 @@ FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j) {
   return keep;
 }
 
-// Summary of the ids of kSumRows consecutive rows (written by the mask plan).
-//   query side: lo/hi = min/max over rows with eq < 0 (lo > hi if none),
-//               glob  = 1 if any row has eq >= 0
-//   key side  : lo/hi = min/max over all keys of the tile
+// ---------------------------------------------------------------------------
+// Mask plan.  With document ids the query rows of one (batch, head) are split
+// into LOCAL rows (eq < 0: see only keys with the same id) and GLOBAL rows
+// (eq >= 0: see every key), each group kept in ascending row order:
+//   perm[0 .. nL)            local rows            (padded with -1 up to nLp,
+//   perm[nLp .. nLp + nG)    global rows            nLp = nL rounded up to 128)
+// Query-side tiles are tiles of this permuted order, so a tile is either all
+// local (it only needs the key tiles whose id interval meets its own) or all
+// global (no doc test at all, plain causal structure).  Keys stay in natural
+// order.  One IdSummary describes 64 consecutive entries of either side.
+// ---------------------------------------------------------------------------
 struct IdSummary {
-  int lo, hi, glob, pad;
+  int lo, hi;      // min / max id: query side over local rows (lo > hi if none), key side over all keys
+  int glob;        // query side: 1 if the tile holds global rows
+  int rmin, rmax;  // query side: smallest / largest original row index of the tile (rmax = -1 if empty)
+  int nvalid;      // query side: rows of the tile that exist
+  int pad0, pad1;
+};
+
+struct QHeader {
+  int nL, nG, nLp, nT128;  // nT128: 128-row tiles of the permuted order that hold rows
 };
 
 // A tile pair can hold a kept element only if a global query row exists or the
@@ -153,10 +168,12 @@ struct KArgs {
   void* dk;
   void* dv;
   float* delta;
-  const int* eq32;        // [B, Hq', Mp]
+  const int* eq32;        // [B, Hq', Mp]   ids in natural row order
   const int* ek32;        // [B, Hk', Np]
-  const IdSummary* qsum;  // [B, Hq', nQs]
-  const IdSummary* ksum;  // [B, Hk', nKs]
+  const int* perm;        // [B, Hq', Pp]   permuted order -> original row (or -1)
+  const QHeader* qhdr;    // [B, Hq']
+  const IdSummary* qsum;  // [B, Hq', nQs]  per 64 entries of the permuted order
+  const IdSummary* ksum;  // [B, Hk', nKs]  per 64 keys
   int64_t q_bs, q_hs, q_rs;
   int64_t k_bs, k_hs, k_rs;
   int64_t v_bs, v_hs, v_rs;
@@ -167,9 +184,12 @@ struct KArgs {
   int64_t dv_bs, dv_hs, dv_rs;
   int64_t eq_bs, eq_hs;   // strides of eq32 (head stride 0 when shared)
   int64_t ek_bs, ek_hs;
+  int64_t pm_bs, pm_hs;   // strides of perm
+  int64_t qh_bs, qh_hs;   // strides of qhdr in entries
   int64_t qs_bs, qs_hs;   // strides of qsum in entries
   int64_t ks_bs, ks_hs;
   int B, H, Hk, G, M, N, gap;
+  int Pp;                 // entries of the permuted order per (b, h)
   int nQs, nKs;           // summary entries per (b, h)
   float scale;            // sm_scale
   float scale_log2e;      // sm_scale * log2(e)
@@ -179,22 +199,26 @@ struct KArgs {
 struct WsLayout {
   int Hq1, Hk1;           // heads stored for eq / ek (1 when the head stride is 0)
   int Mp, Np;             // M, N rounded up to kSumRows
+  int Pp;                 // length of the permuted order
   int nQs, nKs;
-  uint64_t off_eq32, off_ek32, off_qsum, off_ksum, total;  // bytes
+  uint64_t off_eq32, off_ek32, off_perm, off_qhdr, off_qsum, off_ksum, total;  // bytes
 };
 
 inline WsLayout ws_layout(const fa_params* p) {
   WsLayout w;
   w.Hq1 = (p->eq_stride[1] == 0) ? 1 : p->H;
   w.Hk1 = (p->ek_stride[1] == 0) ? 1 : p->H;
-  w.nQs = (p->M + kSumRows - 1) / kSumRows;
+  w.Mp = (p->M + kSumRows - 1) / kSumRows * kSumRows;
   w.nKs = (p->N + kSumRows - 1) / kSumRows;
-  w.Mp = w.nQs * kSumRows;
   w.Np = w.nKs * kSumRows;
+  w.Pp = (p->M + 127) / 128 * 128 + 128;
+  w.nQs = w.Pp / kSumRows;
   uint64_t o = 0;
   auto take = [&](uint64_t bytes) { uint64_t r = o; o += (bytes + 255) & ~uint64_t(255); return r; };
   w.off_eq32 = take(uint64_t(p->B) * w.Hq1 * w.Mp * 4);
   w.off_ek32 = take(uint64_t(p->B) * w.Hk1 * w.Np * 4);
+  w.off_perm = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
+  w.off_qhdr = take(uint64_t(p->B) * w.Hq1 * sizeof(QHeader));
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
   w.total = o;
