@@ -83,7 +83,7 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
     lse = torch.empty(w.B, w.H, w.Lq, device=dev, dtype=torch.float32)
     delta = torch.empty_like(lse)
     dq = torch.empty_like(q)
-    dk = torch.empty(w.B, w.H, w.Lk, w.D, device=dev, dtype=q.dtype)
+    dk = torch.empty(w.B, w.Hk, w.Lk, w.D, device=dev, dtype=q.dtype)
     dv = torch.empty_like(dk)
     p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
     p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()

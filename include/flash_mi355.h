@@ -22,8 +22,9 @@
  *
  * Tensor conventions (identical to the reference, flash_triton.py:27-36):
  *   q, o, dout, dq : [B, H,  M, D]      k, v : [B, Hk, N, D]   (H % Hk == 0)
- *   dk, dv         : [B, H,  N, D]      per *query* head (flash_triton.py:594-595);
- *                                       the caller sums over the group when Hk < H
+ *   dk, dv         : [B, Hk, N, D]      already summed over the query heads of each
+ *                                       group (the reference writes [B,H,N,D] and
+ *                                       sums afterwards, flash_triton.py:594-595,635-637)
  *   lse, delta     : [B, H, M] float32, contiguous.  lse is in log2 units
  *                    (m + log2(l), flash_triton.py:133); -inf for a row with
  *                    no unmasked key
@@ -79,8 +80,8 @@ typedef struct fa_params {
   /* backward operands */
   const void* dout;
   void*       dq;
-  void*       dk;         /* [B,H,N,D] */
-  void*       dv;         /* [B,H,N,D] */
+  void*       dk;         /* [B,Hk,N,D] */
+  void*       dv;         /* [B,Hk,N,D] */
   float*      delta;      /* [B,H,M] */
   /* flexible-mask ids */
   const void* eq;
@@ -134,7 +135,7 @@ int fa_fwd(const fa_params* p, void* stream);
 /* delta = rowsum(o * dout). */
 int fa_bwd_delta(const fa_params* p, void* stream);
 
-/* dk, dv per query head (needs lse, delta). */
+/* dk, dv summed over each group's query heads (needs lse, delta). */
 int fa_bwd_dkdv(const fa_params* p, void* stream);
 
 /* dq (needs lse, delta). */

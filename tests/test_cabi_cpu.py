@@ -1,0 +1,121 @@
+"""Host-side checks that need no GPU: the shared library loads, exports every symbol the header
+declares, agrees with the Python binding on the struct layout, and fa_validate returns the
+documented code for each malformed argument.  The operator's Python layer raises the same
+AssertionErrors as the reference (flash_triton.py:510-530) before touching the GPU."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from flash_mi355 import _cabi, attention, SCORE_FUNC_MODE1_DOC
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / "include" / "flash_mi355.h").read_text()
+
+
+def _declared_functions():
+    body = HEADER.split('extern "C" {')[1]
+    return sorted(set(re.findall(r"^\s*(?:const\s+)?[a-z_0-9]+\*?\s+(fa_[a-z_0-9]+)\s*\(", body, re.M)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _cabi.lib()
+    names = _declared_functions()
+    assert set(names) == set(_cabi.EXPORTS), (names, _cabi.EXPORTS)
+    for n in names:
+        assert getattr(L, n) is not None
+
+
+def test_struct_layout_and_version():
+    L = _cabi.lib()
+    assert L.fa_version() == _cabi.FA_ABI_VERSION == int(re.search(r"#define FA_ABI_VERSION (\d+)", HEADER).group(1))
+    assert L.fa_params_size() == ctypes.sizeof(_cabi.FaParams)
+    for code in range(0, -11, -1):
+        assert L.fa_error_string(code)
+
+
+def _good_params(buf):
+    p = _cabi.FaParams()
+    base = (ctypes.addressof(buf) + 255) & ~255
+    for f in ("q", "k", "v", "o", "lse", "dout", "dq", "dk", "dv", "delta"):
+        setattr(p, f, base)
+    p.B, p.H, p.Hk, p.M, p.N, p.D = 1, 4, 2, 128, 256, 64
+    for f in ("q_stride", "o_stride", "do_stride", "dq_stride"):
+        arr = getattr(p, f); arr[0], arr[1], arr[2], arr[3] = 4 * 128 * 64, 128 * 64, 64, 1
+    for f in ("k_stride", "v_stride", "dk_stride", "dv_stride"):
+        arr = getattr(p, f); arr[0], arr[1], arr[2], arr[3] = 4 * 256 * 64, 256 * 64, 64, 1
+    p.causal, p.score_mode, p.dtype, p.sm_scale = 1, 0, _cabi.FA_DTYPE_BF16, 0.125
+    return p
+
+
+def test_validate_codes():
+    L = _cabi.lib()
+    buf = ctypes.create_string_buffer(4096)
+    v = lambda p, stage=1: L.fa_validate(ctypes.byref(p), stage)
+    assert v(_good_params(buf)) == 0
+    assert L.fa_validate(None, 0) == -1
+    p = _good_params(buf); p.D = 48; assert v(p) == -2           # flash_triton.py:512
+    p = _good_params(buf); p.D = 256; assert v(p) == -2
+    p = _good_params(buf); p.dtype = 5; assert v(p) == -3
+    p = _good_params(buf); p.H = 3; assert v(p) == -4             # H % Hk, flash_triton.py:518
+    p = _good_params(buf); p.M, p.N = 256, 128; assert v(p) == -4  # causal needs N >= M, flash_triton.py:520
+    p = _good_params(buf); p.M, p.N, p.causal = 256, 128, 0; assert v(p) == 0
+    p = _good_params(buf); p.B = 0; assert v(p) == -4
+    p = _good_params(buf); p.q += 8; assert v(p) == -5
+    p = _good_params(buf); p.q_stride[2] = 68; assert v(p) == -5
+    p = _good_params(buf); p.k_stride[3] = 2; assert v(p) == -6
+    p = _good_params(buf); p.score_mode = 3; assert v(p) == -7
+    p = _good_params(buf); p.score_mode = 1; assert v(p) == -7     # doc mode without ids
+    p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
+    p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
+    p = _good_params(buf); p.flags = 1; assert v(p) == -7
+
+
+def test_workspace_size():
+    L = _cabi.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = _good_params(buf)
+    assert L.fa_workspace_bytes(ctypes.byref(p)) == 0
+    p.score_mode = 1
+    p.eq_stride[0], p.eq_stride[1], p.eq_stride[2] = 128, 0, 1       # ids shared by the heads
+    p.ek_stride[0], p.ek_stride[1], p.ek_stride[2] = 4 * 256, 256, 1   # per head
+    r256 = lambda x: (x + 255) // 256 * 256
+    Pp = 128 + 128
+    want = r256(128 * 4) + r256(4 * 256 * 4) + r256(Pp * 4) + r256(16) + r256(Pp // 64 * 32) + r256(4 * 4 * 32)
+    assert L.fa_workspace_bytes(ctypes.byref(p)) == want
+
+
+def test_python_layer_asserts_like_the_reference():
+    q = torch.zeros(1, 4, 8, 64, dtype=torch.bfloat16)
+    k = torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16)
+    e_q = torch.zeros(1, 4, 8, dtype=torch.int32)
+    with pytest.raises(AssertionError):
+        attention(q, k, torch.zeros(1, 2, 16, 32, dtype=torch.bfloat16))          # feature sizes differ
+    with pytest.raises(AssertionError):
+        attention(torch.zeros(1, 4, 8, 48), torch.zeros(1, 2, 16, 48), torch.zeros(1, 2, 16, 48))   # D not in {16,32,64,128}
+    with pytest.raises(AssertionError):
+        attention(q, k, torch.zeros(1, 1, 16, 64, dtype=torch.bfloat16))          # kv head counts differ
+    with pytest.raises(AssertionError):
+        attention(torch.zeros(1, 3, 8, 64), k, k)                                   # H % Hk
+    with pytest.raises(AssertionError):
+        attention(torch.zeros(1, 4, 32, 64, dtype=torch.bfloat16), k, k, causal=True)   # causal with N < M
+    with pytest.raises(AssertionError):
+        attention(q, k, k, eq=e_q)                                                  # eq without ek
+    with pytest.raises(AssertionError):
+        attention(q, k, k, score_func_mode=SCORE_FUNC_MODE1_DOC)                    # doc mode without ids
+    with pytest.raises(AssertionError):
+        attention(q, k, k)                                                          # CPU tensors: no CPU fallback
+
+
+def test_drop_in_module_name():
+    import flash_triton
+    import flash_mi355
+    assert flash_triton.attention is flash_mi355.attention
+    assert flash_triton.FlashAttention is flash_mi355.FlashAttention
+    assert (flash_triton.SCORE_FUNC_MODE0_NOPE, flash_triton.SCORE_FUNC_MODE1_DOC) == (0, 1)
+    import inspect
+    sig = inspect.signature(flash_triton.attention)
+    assert list(sig.parameters) == ["q", "k", "v", "causal", "sm_scale", "eq", "ek", "score_func_mode"]
+    assert [p.default for p in sig.parameters.values()][3:] == [False, None, None, None, 0]

@@ -95,6 +95,9 @@ CASES = [
     (1, 2, 2, 77, 333, 64, torch.bfloat16, True, True),        # ragged + rectangular
     (1, 2, 2, 256, 256, 32, torch.bfloat16, True, True),
     (1, 1, 1, 1024, 1024, 128, torch.bfloat16, True, True),
+    (1, 2, 2, 256, 256, 16, torch.bfloat16, True, True),
+    (2, 2, 1, 100, 300, 16, torch.float16, True, True),
+    (1, 2, 2, 192, 192, 64, torch.bfloat16, False, False),
 ]
 
 
@@ -127,3 +130,83 @@ def test_all_global_and_all_local_ids():
 
 def test_per_head_int64_ids():
     _run_case(1, 3, 3, 192, 192, 64, torch.bfloat16, True, True, seed=9, per_head_ids=True, id_dtype=torch.int64)
+
+
+def test_golden_fixtures():
+    """The committed fixtures (inputs + fp64 answers) through the HIP operator."""
+    from pathlib import Path
+    from flash_mi355 import attention, attention_with_lse, mask_dump
+    for path in sorted((Path(__file__).parent / "golden").glob("*.npz")):
+        z = np.load(path, allow_pickle=False)
+        dt = torch.bfloat16 if "bfloat16" in str(z["dtype"]) else torch.float16
+        causal, doc = bool(z["causal"]), bool(z["doc"])
+        print("fixture", path.stem, flush=True)
+        q, k, v, do = (torch.from_numpy(z[n]).to(dt).cuda() for n in ("q", "k", "v", "do"))
+        eq = torch.from_numpy(z["eq"]).cuda() if doc else None
+        ek = torch.from_numpy(z["ek"]).cuda() if doc else None
+        mode = 1 if doc else 0
+        B, H, M, _ = q.shape
+        N = k.shape[2]
+        keep = np.unpackbits(z["keep"], axis=-1, count=N).astype(bool)
+        assert np.array_equal(mask_dump(B, H, M, N, causal, eq, ek, mode).cpu().numpy(), keep)
+        out, lse = attention_with_lse(q, k, v, causal, None, eq, ek, mode)
+        assert (out.float().cpu().numpy() - z["o"]).__abs__().max() <= TOL_O
+        assert np.abs(lse.cpu().numpy() - z["lse"]).max() <= TOL_LSE
+        q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+        attention(q, k, v, causal, None, eq, ek, mode).backward(do)
+        for name, got in (("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
+            ref = z[name]
+            assert np.abs(got.float().cpu().numpy() - ref).max() <= TOL_O * max(1.0, np.abs(ref).max() / 4), name
+
+
+def test_device_mask_plan_matches_host_restatement():
+    """Workspace written by fa_mask_plan against tests/_plan_ref.py."""
+    import ctypes
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan
+    from tests import _plan_ref as P
+    rng = np.random.default_rng(3)
+    B, H, M, N, D = 2, 2, 300, 450, 64
+    ek = np.stack([_ids(rng, B, H, N, "uniform") for _ in range(H)], axis=1)
+    eq = np.ascontiguousarray(ek[:, :, N - M:])
+    q = torch.zeros(B, H, M, D, dtype=torch.bfloat16, device="cuda")
+    k = torch.zeros(B, H, N, D, dtype=torch.bfloat16, device="cuda")
+    plan = _Plan(q, k, k, True, 1.0, torch.from_numpy(eq).cuda(), torch.from_numpy(ek).cuda(), 1)
+    plan.ensure_workspace(q.device)
+    torch.cuda.synchronize()
+    ws = plan.workspace.cpu().numpy()
+    r256 = lambda x: (x + 255) // 256 * 256
+    Mp, Np, Pp = (M + 63) // 64 * 64, (N + 63) // 64 * 64, (M + 127) // 128 * 128 + 128
+    nQs, nKs = Pp // 64, Np // 64
+    off = 0
+    take = lambda n: (off, off + n)
+    o_eq = off; off += r256(B * H * Mp * 4)
+    o_ek = off; off += r256(B * H * Np * 4)
+    o_pm = off; off += r256(B * H * Pp * 4)
+    o_hd = off; off += r256(B * H * 16)
+    o_qs = off; off += r256(B * H * nQs * 32)
+    o_ks = off; off += r256(B * H * nKs * 32)
+    assert off == ws.size
+    i32 = lambda o, n: ws[o:o + 4 * n].view(np.int32)
+    perm = i32(o_pm, B * H * Pp).reshape(B, H, Pp)
+    hdr = i32(o_hd, B * H * 4).reshape(B, H, 4)
+    qs = i32(o_qs, B * H * nQs * 8).reshape(B, H, nQs, 8)
+    ks = i32(o_ks, B * H * nKs * 8).reshape(B, H, nKs, 8)
+    assert np.array_equal(i32(o_eq, B * H * Mp).reshape(B, H, Mp)[:, :, :M], eq)
+    assert np.array_equal(i32(o_ek, B * H * Np).reshape(B, H, Np)[:, :, :N], ek)
+    for b in range(B):
+        for h in range(H):
+            rp, rh, rq = P.plan_q(eq[b, h].astype(np.int64), M)
+            assert np.array_equal(perm[b, h], rp)
+            assert list(hdr[b, h]) == [rh["nL"], rh["nG"], rh["nLp"], rh["nT128"]]
+            for t, s_ in enumerate(rq):
+                got = qs[b, h, t]
+                assert got[5] == s_["nvalid"] and got[2] == s_["glob"] and got[4] == s_["rmax"]
+                if s_["nvalid"]:
+                    assert got[3] == s_["rmin"]
+                if s_["lo"] <= s_["hi"]:
+                    assert (got[0], got[1]) == (s_["lo"], s_["hi"])
+                else:
+                    assert got[0] > got[1]
+            for t, s_ in enumerate(P.plan_k(ek[b, h].astype(np.int64), N)):
+                assert (ks[b, h, t, 0], ks[b, h, t, 1]) == (s_["lo"], s_["hi"])

@@ -1,0 +1,235 @@
+"""Pins the CPU oracle (oracle/attention_oracle.py) without any GPU: brute force on
+tiny inputs, library routines for special cases, closed-form invariants and fp64
+gradcheck.  Each check is chosen so that a plausible slip (dropped term, wrong sign
+or index, transposed operand, wrong causal alignment) fails at least one of them."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attention_oracle as O
+
+
+def _rand(B, H, M, N, D, Hk=None, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    Hk = Hk or H
+    return (torch.randn(B, H, M, D, generator=g, dtype=dtype), torch.randn(B, Hk, N, D, generator=g, dtype=dtype),
+            torch.randn(B, Hk, N, D, generator=g, dtype=dtype), torch.randn(B, H, M, D, generator=g, dtype=dtype))
+
+
+def _ids(rng, B, H, L, p_new=0.15, p_glob=0.1):
+    ids = -(np.cumsum(rng.random((B, H, L)) < p_new, axis=-1) + 1)
+    ids[rng.random((B, H, L)) < p_glob] = rng.integers(0, 3)
+    return ids.astype(np.int64)
+
+
+# ------------------------------------------------------------------ mask
+@pytest.mark.parametrize("M,N,causal", [(7, 7, True), (5, 11, True), (9, 4, False), (6, 6, False), (1, 8, True)])
+def test_mask_brute_force(M, N, causal):
+    rng = np.random.default_rng(M * 100 + N)
+    B, H = 2, 3
+    eq, ek = _ids(rng, B, H, M), _ids(rng, B, H, N)
+    got = np.broadcast_to(O.keep_mask(M, N, causal, eq, ek, 1), (B, H, M, N))
+    gap = max(0, N - M)
+    for b in range(B):
+        for h in range(H):
+            for i in range(M):
+                for j in range(N):
+                    want = (not causal or gap + i >= j) and (eq[b, h, i] >= 0 or eq[b, h, i] == ek[b, h, j])
+                    assert got[b, h, i, j] == want
+    plain = np.broadcast_to(O.keep_mask(M, N, causal), (1, 1, M, N))
+    for i in range(M):
+        for j in range(N):
+            assert plain[0, 0, i, j] == (not causal or gap + i >= j)
+
+
+def test_mask_special_cases():
+    L = 12
+    # every query global: the doc test never removes anything
+    eq = np.zeros((1, 1, L), np.int64)
+    ek = -np.arange(1, L + 1)[None, None]
+    assert np.array_equal(O.keep_mask(L, L, True, eq, ek, 1), O.keep_mask(L, L, True))
+    assert O.keep_mask(L, L, False, eq, ek, 1).all()
+    # packed documents, all local, eq == ek: block diagonal
+    ids = -np.repeat(np.arange(1, 4), 4)[None, None]
+    blk = O.keep_mask(L, L, False, ids, ids, 1)[0, 0]
+    want = np.kron(np.eye(3, dtype=bool), np.ones((4, 4), bool))
+    assert np.array_equal(blk, want)
+    # bottom-right alignment: rectangular causal == last M rows of the square N x N causal mask
+    M, N = 5, 9
+    assert np.array_equal(O.keep_mask(M, N, True)[0, 0], O.keep_mask(N, N, True)[0, 0][N - M:])
+    # reference sampler identity (testing.py:114-117): (eq>=0)|(eq==eq^T) & tril for self attention
+    rng = np.random.default_rng(3)
+    e = _ids(rng, 1, 1, L)
+    t = torch.from_numpy(e[0, 0])
+    ref = ((t[:, None] >= 0) | (t[:, None] == t[None, :])) & (torch.arange(L)[:, None] >= torch.arange(L)[None, :])
+    assert np.array_equal(O.keep_mask(L, L, True, e, e, 1)[0, 0], ref.numpy())
+
+
+def test_unknown_mode_rejected():
+    with pytest.raises(ValueError):
+        O.keep_mask(4, 4, False, np.zeros((1, 1, 4)), np.zeros((1, 1, 4)), 7)
+
+
+# ------------------------------------------------------------------ forward
+@pytest.mark.parametrize("M,N,causal,doc", [(16, 16, False, False), (16, 16, True, False), (8, 24, True, False),
+                                             (16, 16, True, True), (8, 24, True, True), (24, 8, False, True)])
+def test_forward_against_sdpa_and_logsumexp(M, N, causal, doc):
+    B, H, D = 2, 2, 8
+    q, k, v, _ = _rand(B, H, M, N, D, seed=M + N)
+    rng = np.random.default_rng(M * N)
+    eq = ek = None
+    mode = 0
+    if doc:
+        mode = 1
+        ek_np = _ids(rng, B, H, N)
+        eq_np = ek_np[..., N - M:] if N >= M else _ids(rng, B, H, M)
+        eq_np = eq_np.copy(); eq_np[..., 0] = 0   # keep every row non-empty for the library comparison
+        eq, ek = torch.from_numpy(eq_np), torch.from_numpy(ek_np)
+    o, lse = O.attention_closed_form(q, k, v, causal, None, eq, ek, mode, dtype=torch.float64)
+    # independent route: boolean mask built with torch ops, library SDPA + library logsumexp
+    gap = max(0, N - M)
+    keep = torch.ones(B, H, M, N, dtype=torch.bool)
+    if causal:
+        keep &= (torch.arange(M)[:, None] + gap) >= torch.arange(N)[None, :]
+    if doc:
+        keep &= (eq[..., :, None] >= 0) | (eq[..., :, None] == ek[..., None, :])
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=keep)
+    s = (q @ k.transpose(-1, -2)) / math.sqrt(D)
+    ref_lse = torch.logsumexp(s.masked_fill(~keep, float("-inf")), -1)
+    assert torch.allclose(o, ref, atol=1e-12)
+    assert torch.allclose(lse, ref_lse, atol=1e-12)
+    if causal and M == N and not doc:
+        assert torch.allclose(o, F.scaled_dot_product_attention(q, k, v, is_causal=True), atol=1e-12)
+
+
+def test_sm_scale_argument():
+    q, k, v, _ = _rand(1, 1, 6, 6, 4)
+    o1, _ = O.attention_closed_form(q, k, v, False, 0.37, dtype=torch.float64)
+    ref = torch.softmax((q @ k.transpose(-1, -2)) * 0.37, -1) @ v
+    assert torch.allclose(o1, ref, atol=1e-12)
+
+
+def test_block_diagonal_invariance():
+    """Rows of a local document equal attention over that document alone."""
+    B, H, L, D = 1, 2, 20, 8
+    q, k, v, _ = _rand(B, H, L, L, D, seed=5)
+    bounds = [0, 6, 13, 20]
+    ids = np.zeros(L, np.int64)
+    for d, (a, b) in enumerate(zip(bounds[:-1], bounds[1:])):
+        ids[a:b] = -(d + 1)
+    e = torch.from_numpy(ids)[None, None].expand(B, H, L)
+    o, lse = O.attention_closed_form(q, k, v, True, None, e, e, 1, dtype=torch.float64)
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        o_doc, lse_doc = O.attention_closed_form(q[:, :, a:b], k[:, :, a:b], v[:, :, a:b], True, dtype=torch.float64)
+        assert torch.allclose(o[:, :, a:b], o_doc, atol=1e-12)
+        assert torch.allclose(lse[:, :, a:b], lse_doc, atol=1e-12)
+
+
+def test_rows_are_convex_combinations():
+    q, k, v, _ = _rand(1, 2, 10, 14, 4, seed=2)
+    v = v.abs()
+    o, _ = O.attention_closed_form(q, k, v, True, dtype=torch.float64)
+    assert (o >= v.min(dim=2, keepdim=True).values - 1e-12).all()
+    assert (o <= v.max(dim=2, keepdim=True).values + 1e-12).all()
+
+
+def test_empty_rows_convention():
+    """A row with no kept key: O = 0, LSE = -inf, zero gradient contributions."""
+    B, H, L, D = 1, 1, 6, 4
+    q, k, v, do = _rand(B, H, L, L, D, seed=9)
+    eq = torch.tensor([-1, -1, -5, -2, -2, 0])[None, None]
+    ek = torch.tensor([-1, -1, -9, -2, -2, -3])[None, None]   # row 2 (id -5) matches nothing
+    o, lse, delta, dq, dk, dv = O.attention_grads(q, k, v, do, False, None, eq, ek, 1)
+    assert torch.isinf(lse[0, 0, 2]) and lse[0, 0, 2] < 0
+    assert (o[0, 0, 2] == 0).all() and (dq[0, 0, 2] == 0).all()
+    assert not torch.isnan(o).any() and not torch.isnan(dk).any() and not torch.isnan(dv).any()
+    # dropping the dead row changes nothing for the key/value gradients
+    keep_rows = [0, 1, 3, 4, 5]
+    _, _, _, _, dk2, dv2 = O.attention_grads(q[:, :, keep_rows], k, v, do[:, :, keep_rows], False, None,
+                                             eq[:, :, keep_rows], ek, 1)
+    assert torch.allclose(dk, dk2, atol=1e-12) and torch.allclose(dv, dv2, atol=1e-12)
+
+
+# ------------------------------------------------------------------ gradients
+@pytest.mark.parametrize("M,N,causal,doc,Hk", [(6, 6, True, True, 2), (4, 9, True, True, 2), (7, 5, False, False, 2),
+                                                (6, 6, True, True, 1)])
+def test_explicit_gradients_against_autograd_of_sdpa(M, N, causal, doc, Hk):
+    B, H, D = 1, 2, 4
+    q, k, v, do = _rand(B, H, M, N, D, Hk=Hk, seed=M * 7 + N)
+    rng = np.random.default_rng(11)
+    eq = ek = None
+    mode = 0
+    if doc:
+        mode = 1
+        ek_np = _ids(rng, B, H, N)
+        eq_np = ek_np[..., N - M:].copy()
+        eq_np[..., 0] = 0
+        eq, ek = torch.from_numpy(eq_np), torch.from_numpy(ek_np)
+    o, lse, delta, dq, dk, dv = O.attention_grads(q, k, v, do, causal, None, eq, ek, mode)
+    # independent route: autograd through the library SDPA with an explicit mask
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    gap = max(0, N - M)
+    keep = torch.ones(B, H, M, N, dtype=torch.bool)
+    if causal:
+        keep &= (torch.arange(M)[:, None] + gap) >= torch.arange(N)[None, :]
+    if doc:
+        keep &= (eq[..., :, None] >= 0) | (eq[..., :, None] == ek[..., None, :])
+    G = H // Hk
+    ref = F.scaled_dot_product_attention(qa, ka.repeat_interleave(G, 1), va.repeat_interleave(G, 1), attn_mask=keep)
+    ref.backward(do)
+    assert torch.allclose(o, ref.detach(), atol=1e-12)
+    assert torch.allclose(dq, qa.grad, atol=1e-11)
+    assert torch.allclose(dk, ka.grad, atol=1e-11)      # includes the grouped-query sum
+    assert torch.allclose(dv, va.grad, atol=1e-11)
+    assert torch.allclose(delta, (o * do).sum(-1), atol=1e-12)
+    # and the oracle's own autograd route
+    o2, lse2, dq2, dk2, dv2 = O.attention_autograd(q, k, v, do, causal, None, eq, ek, mode, dtype=torch.float64)
+    for a_, b_ in ((dq, dq2), (dk, dk2), (dv, dv2), (lse, lse2)):
+        assert torch.allclose(a_, b_, atol=1e-11)
+
+
+def test_gradcheck_closed_form():
+    B, H, M, N, D = 1, 1, 4, 6, 3
+    q, k, v, _ = _rand(B, H, M, N, D, seed=4)
+    eq = torch.tensor([0, -1, -2, -2])[None, None]
+    ek = torch.tensor([-1, -1, -2, -2, -3, -2])[None, None]
+    fn = lambda q_, k_, v_: O.attention_closed_form(q_, k_, v_, True, None, eq, ek, 1, dtype=torch.float64)[0]
+    assert torch.autograd.gradcheck(fn, tuple(t.requires_grad_(True) for t in (q, k, v)), eps=1e-6, atol=1e-5)
+
+
+# ------------------------------------------------------------------ tiled restatement
+@pytest.mark.parametrize("M,N,causal,doc,Hk,bm,bn", [(20, 20, True, True, 2, 8, 8), (9, 23, True, True, 1, 4, 8),
+                                                      (17, 12, False, False, 2, 8, 4), (16, 16, True, False, 2, 16, 16)])
+def test_tiled_kernels_equal_closed_form(M, N, causal, doc, Hk, bm, bn):
+    B, H, D = 1, 2, 4
+    q, k, v, do = _rand(B, H, M, N, D, Hk=Hk, seed=M + 3 * N)
+    rng = np.random.default_rng(M)
+    eq = ek = None
+    mode = 0
+    if doc:
+        mode = 1
+        ek = _ids(rng, B, H, N)
+        eq = ek[..., N - M:]
+    scale = 1.0 / math.sqrt(D)
+    Ot, L2, dQ, dK, dV = O.attention_tiled(q.numpy(), k.numpy(), v.numpy(), do.numpy(), causal, scale, eq, ek, mode, bm, bn)
+    te = (lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)))
+    o, lse, delta, dq, dk, dv = O.attention_grads(q, k, v, do, causal, scale, te(eq), te(ek), mode)
+    assert np.allclose(Ot, o.numpy(), atol=1e-12)
+    assert np.allclose(L2 / O.LOG2E, lse.numpy(), atol=1e-12)       # the kernel stores log2 units
+    assert np.allclose(dQ, dq.numpy(), atol=1e-11)
+    assert np.allclose(dK, dk.numpy(), atol=1e-11)
+    assert np.allclose(dV, dv.numpy(), atol=1e-11)
+
+
+def test_eager_cpu_path_matches_closed_form():
+    B, H, M, N, D = 1, 2, 12, 20, 8
+    q, k, v, _ = _rand(B, H, M, N, D, seed=8, dtype=torch.float32)
+    rng = np.random.default_rng(8)
+    ek = torch.from_numpy(_ids(rng, B, H, N)); eq = ek[..., N - M:].clone(); eq[..., 0] = 0
+    keep = (eq[..., :, None] >= 0) | (eq[..., :, None] == ek[..., None, :])
+    got = O.eager_attention_cpu(q, k, v, True, keep)
+    ref, _ = O.attention_closed_form(q, k, v, True, None, eq, ek, 1)
+    assert torch.allclose(got, ref, atol=1e-5)

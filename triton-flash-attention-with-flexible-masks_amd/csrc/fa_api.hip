@@ -9,8 +9,11 @@ static thread_local int g_last_hip_error = 0;
 
 static bool d_supported(int D) { return D == 16 || D == 32 || D == 64 || D == 128; }
 
-static int check_tensor(const void* ptr, const int64_t* st) {
+// rows/D: extent of one (batch, head) slice; the kernels address a slice through a
+// buffer resource whose byte range must stay below 2 GiB
+static int check_tensor(const void* ptr, const int64_t* st, int rows, int D) {
   if (ptr == nullptr) return FA_ERR_NULLPTR;
+  if (st[2] < 0 || (int64_t(rows - 1) * st[2] + D) * 2 >= (int64_t(1) << 31)) return FA_ERR_NOT_IMPLEMENTED;
   if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0) return FA_ERR_ALIGN;
   if (st[3] != 1) return FA_ERR_STRIDE;
   if ((st[0] % 8) != 0 || (st[1] % 8) != 0 || (st[2] % 8) != 0) return FA_ERR_ALIGN;
@@ -56,16 +59,16 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   }
   if (stage == 2) return FA_OK;
   int rc;
-  if ((rc = check_tensor(p->q, p->q_stride)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->k, p->k_stride)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->v, p->v_stride)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->o, p->o_stride)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->q, p->q_stride, p->M, p->D)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->k, p->k_stride, p->N, p->D)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->v, p->v_stride, p->N, p->D)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->o, p->o_stride, p->M, p->D)) != FA_OK) return rc;
   if (p->lse == nullptr) return FA_ERR_NULLPTR;
   if (stage == 1) {
-    if ((rc = check_tensor(p->dout, p->do_stride)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dq, p->dq_stride)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dk, p->dk_stride)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dv, p->dv_stride)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dout, p->do_stride, p->M, p->D)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dq, p->dq_stride, p->M, p->D)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dk, p->dk_stride, p->N, p->D)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dv, p->dv_stride, p->N, p->D)) != FA_OK) return rc;
     if (p->delta == nullptr) return FA_ERR_NULLPTR;
   }
   return FA_OK;

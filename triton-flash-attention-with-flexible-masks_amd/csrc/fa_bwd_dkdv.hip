@@ -16,8 +16,8 @@
 // order of the mask plan: tiles are gathered row by row through the permutation,
 // and only tiles whose id interval and row range can meet this workgroup's keys
 // are visited.
-// dK, dV are written per query head; the group sum for grouped-query attention is
-// done by the caller (flash_triton.py:635-637).
+// The query heads of a grouped-query group are walked inside the kernel, so dK, dV are
+// written once, already summed (the reference sums afterwards, flash_triton.py:635-637).
 
 #include "fa_tile.h"
 
@@ -29,29 +29,29 @@ void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
   using vec8 = typename E::vec8;
-  constexpr int BK = 128, BQ = 64, KS = D / 16, DBN = D / 32;
-  constexpr int TILE_BYTES = BQ * D * 2;
+  constexpr int BK = 128, BQ = 64, KS = D / 16;
+  constexpr int DL = D < 32 ? 32 : D;  // LDS row width: D = 16 is staged as 32 columns, the upper 16 zero
+  constexpr int DBN = DL / 32;
+  constexpr int TILE_BYTES = BQ * DL * 2;
   constexpr int AUX_OFF = 4 * TILE_BYTES;  // [2 buffers][4 arrays][64] x 4 bytes
   constexpr int AUX_BYTES = 1024;
-  using Loader = TileLoader<D, BQ>;
+  using Loader = TileLoader<DL, BQ, D>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lq = lane & 31, g = lane >> 5;
 
+  // one workgroup per (key tile, batch, kv head); the query heads of the group are walked in
+  // turn with K/V staying in registers, so dK/dV leave the kernel already summed over the group
   const int nKt = (a.N + BK - 1) / BK;
-  int kt, bh;
-  if (!block_to_tile(nKt, a.B * a.H, kt, bh)) return;  // causal: the first key tiles see the most rows
-  const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  int kt, bhk;
+  if (!block_to_tile(nKt, a.B * a.Hk, kt, bhk)) return;  // causal: the first key tiles see the most rows
+  const int b = bhk / a.Hk, hk = bhk % a.Hk;
 
-  const T* qp = reinterpret_cast<const T*>(a.q) + b * a.q_bs + h * a.q_hs;
   const T* kp = reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs;
   const T* vp = reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs;
-  const T* dop = reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs;
-  T* dkp = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + h * a.dk_hs;
-  T* dvp = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + h * a.dv_hs;
-  const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
-  const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+  T* dkp = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs;
+  T* dvp = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs;
 
   const int n0 = kt * BK;
   const int nw = n0 + wave * 32;
@@ -67,51 +67,25 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
   const float c = a.scale_log2e;
 
+  // per query head state (set at the top of the head loop)
+  const float* lsep = nullptr;
+  const float* delp = nullptr;
   int ek_j = 0;
   int wk_lo = 0, wk_hi = 0;   // id interval of this wave's 32 keys
-  int gk_lo = 0, gk_hi = 0;   // of the workgroup's 128 keys
   const int* eqp = nullptr;
   const int* pmp = nullptr;
   const IdSummary* qsum = nullptr;
-  int nQtiles = (a.M + BQ - 1) / BQ;
-  int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
-  if (DOC) {
-    ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
-    eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
-    pmp = a.perm + b * a.pm_bs + h * a.pm_hs;
-    qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
-    const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
-    const IdSummary s0 = ks[n0 / kSumRows];
-    gk_lo = s0.lo; gk_hi = s0.hi;
-    if (n0 / kSumRows + 1 < a.nKs) {
-      const IdSummary s1 = ks[n0 / kSumRows + 1];
-      gk_lo = min(gk_lo, s1.lo); gk_hi = max(gk_hi, s1.hi);
-    }
-    const bool valid = key < a.N;
-    int lo = valid ? ek_j : 0x7fffffff, hi = valid ? ek_j : (int)0x80000000;
-#pragma unroll
-    for (int off = 16; off >= 1; off >>= 1) {
-      lo = min(lo, __shfl_xor(lo, off));
-      hi = max(hi, __shfl_xor(hi, off));
-    }
-    wk_lo = lo; wk_hi = hi;
-    nQtiles = a.nQs;
-    first = 0;
-  }
-  TileIter it;
-  it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000);
 
   Loader ldQ, ldO;
-  ldQ.init(qp, a.q_rs, a.M);
-  ldO.init(dop, a.do_rs, a.M);
-  LdsOffsets<D> lo;
+  LdsOffsets<DL> lo;
   lo.init();
   // gathered loads: byte offset of the lane's chunk inside its row, and the tile rows it fetches
   int g_coff[Loader::PER], g_rit[Loader::PER];
 #pragma unroll
   for (int i = 0; i < Loader::PER; ++i) {
     g_rit[i] = (i * 4 + wave) * Loader::RPI + lane / Loader::CPR;
-    g_coff[i] = ((lane % Loader::CPR) ^ swz<D, SWZ_ROW>(g_rit[i])) * 16;
+    const int gc = (lane % Loader::CPR) ^ swz<DL, SWZ_ROW>(g_rit[i]);
+    g_coff[i] = gc < D / 8 ? gc * 16 : kOobOffset;
   }
 
   f32x16 dk[DBN], dv[DBN];
@@ -176,12 +150,12 @@ void bwd_dkdv_kernel(const KArgs a) {
       f32x16 s = zero, dp = zero;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const vec8 qa = lds_row8<E>(lqt + lo.row[ks] + qb * 32 * D * 2);
+        const vec8 qa = lds_row8<E>(lqt + lo.row[ks] + qb * 32 * DL * 2);
         s = E::mfma32(qa, kf[ks], s);
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const vec8 da = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * D * 2);
+        const vec8 da = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * DL * 2);
         dp = E::mfma32(da, vf[ks], dp);
       }
       // s -> P, dp -> dS for this lane's 16 query rows of the block
@@ -218,7 +192,7 @@ void bwd_dkdv_kernel(const KArgs a) {
           pf[t] = pr[0]; pf[t + 1] = pr[1];
           dsf[t] = dr[0]; dsf[t + 1] = dr[1];
         }
-        const int goff = (2 * qb + half) * 16 * D * 2;
+        const int goff = (2 * qb + half) * 16 * DL * 2;
 #pragma unroll
         for (int db = 0; db < DBN; ++db) {
           const vec8 dot = lds_tr8<E>(ldo + lo.tr[db][0] + goff, ldo + lo.tr[db][1] + goff);
@@ -233,31 +207,69 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
 
-  // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and
-  // the row indices of the tile after that are fetched
-  int cur = it.next();
-  int nxt = cur >= 0 ? it.next() : -1;
-  if (cur >= 0) {
-    if (DOC) fetch_idx(cur);
-    load_tile(cur, 0);
-    if (DOC && nxt >= 0) fetch_idx(nxt);
-  }
-  while (cur >= 0) {
-    int nxt2 = nxt >= 0 ? it.next() : -1;
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) load_tile(nxt, 1);
-    if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-    compute(0, cur);
-    cur = nxt; nxt = nxt2;
-    if (cur < 0) break;
-    nxt2 = nxt >= 0 ? it.next() : -1;
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) load_tile(nxt, 0);
-    if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-    compute(1, cur);
-    cur = nxt; nxt = nxt2;
+  for (int gi = 0; gi < a.G; ++gi) {
+    const int h = hk * a.G + gi;
+    lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
+    delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+    ldQ.init(reinterpret_cast<const T*>(a.q) + b * a.q_bs + h * a.q_hs, a.q_rs, a.M);
+    ldO.init(reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs, a.do_rs, a.M);
+    int gk_lo = 0, gk_hi = 0;   // id interval of the workgroup's 128 keys
+    int nQtiles = (a.M + BQ - 1) / BQ;
+    int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
+    if (DOC) {
+      ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
+      eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
+      pmp = a.perm + b * a.pm_bs + h * a.pm_hs;
+      qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
+      const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
+      const IdSummary s0 = ks[n0 / kSumRows];
+      gk_lo = s0.lo; gk_hi = s0.hi;
+      if (n0 / kSumRows + 1 < a.nKs) {
+        const IdSummary s1 = ks[n0 / kSumRows + 1];
+        gk_lo = min(gk_lo, s1.lo); gk_hi = max(gk_hi, s1.hi);
+      }
+      const bool valid = key < a.N;
+      int lo_ = valid ? ek_j : 0x7fffffff, hi_ = valid ? ek_j : (int)0x80000000;
+#pragma unroll
+      for (int off = 16; off >= 1; off >>= 1) {
+        lo_ = min(lo_, __shfl_xor(lo_, off));
+        hi_ = max(hi_, __shfl_xor(hi_, off));
+      }
+      wk_lo = lo_; wk_hi = hi_;
+      nQtiles = a.nQs;
+      first = 0;
+    }
+    TileIter it;
+    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000);
+    if (gi > 0) __syncthreads();  // the previous head's last tile may still be read from LDS
+
+    // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and
+    // the row indices of the tile after that are fetched
+    int cur = it.next();
+    int nxt = cur >= 0 ? it.next() : -1;
+    if (cur >= 0) {
+      if (DOC) fetch_idx(cur);
+      load_tile(cur, 0);
+      if (DOC && nxt >= 0) fetch_idx(nxt);
+    }
+    while (cur >= 0) {
+      int nxt2 = nxt >= 0 ? it.next() : -1;
+      wait_async_loads();
+      __syncthreads();
+      if (nxt >= 0) load_tile(nxt, 1);
+      if (DOC && nxt2 >= 0) fetch_idx(nxt2);
+      compute(0, cur);
+      cur = nxt; nxt = nxt2;
+      if (cur < 0) break;
+      nxt2 = nxt >= 0 ? it.next() : -1;
+      wait_async_loads();
+      __syncthreads();
+      if (nxt >= 0) load_tile(nxt, 0);
+      if (DOC && nxt2 >= 0) fetch_idx(nxt2);
+      compute(1, cur);
+      cur = nxt; nxt = nxt2;
+    }
+
   }
 
   if (key < a.N) {
@@ -268,6 +280,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
+        if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
         const typename E::vec2 k0 = E::cvt2(dk[db][4 * q4 + 0] * sc, dk[db][4 * q4 + 1] * sc);
         const typename E::vec2 k1 = E::cvt2(dk[db][4 * q4 + 2] * sc, dk[db][4 * q4 + 3] * sc);
         const typename E::vec2 v0 = E::cvt2(dv[db][4 * q4 + 0], dv[db][4 * q4 + 1]);
@@ -285,8 +298,8 @@ template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BK = 128, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const int slots = (a.B * a.H + 7) / 8;
-  const size_t lds = 4 * BQ * D * 2 + 2 * 1024;
+  const int slots = (a.B * a.Hk + 7) / 8;
+  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024;
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -310,6 +323,7 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
     case 128: return launch_cd<Tag, 128>(a, causal, doc, s);
     case 64: return launch_cd<Tag, 64>(a, causal, doc, s);
     case 32: return launch_cd<Tag, 32>(a, causal, doc, s);
+    case 16: return launch_cd<Tag, 16>(a, causal, doc, s);
     default: return -1;
   }
 }

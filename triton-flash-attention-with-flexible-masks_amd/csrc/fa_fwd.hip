@@ -30,8 +30,10 @@ void fwd_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
   using vec8 = typename E::vec8;
-  constexpr int BM = 128, BN = 64, KS = D / 16, DBN = D / 32;
-  constexpr int TILE_BYTES = BN * D * 2;
+  constexpr int BM = 128, BN = 64, KS = D / 16;
+  constexpr int DL = D < 32 ? 32 : D;  // LDS row width: D = 16 is staged as 32 columns, the upper 16 zero
+  constexpr int DBN = DL / 32;
+  constexpr int TILE_BYTES = BN * DL * 2;
   constexpr float RESCALE_THRESH = 8.0f;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -70,10 +72,10 @@ void fwd_kernel(const KArgs a) {
   TileIter it;
   it.init_keys(0, (qc.hi_key(a) + BN - 1) / BN, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
 
-  TileLoader<D, BN> ldK, ldV;
+  TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
   ldV.init(vp, a.v_rs, a.N);
-  LdsOffsets<D> lo;
+  LdsOffsets<DL> lo;
   lo.init();
 
   f32x16 o[DBN];
@@ -101,7 +103,7 @@ void fwd_kernel(const KArgs a) {
       s[kb] = zero;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * D * 2);
+        const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
         s[kb] = E::mfma32(kf, qf[ks], s[kb]);
       }
     }
@@ -166,7 +168,7 @@ void fwd_kernel(const KArgs a) {
       }
 #pragma unroll
       for (int db = 0; db < DBN; ++db) {
-        const vec8 vf = lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * D * 2, lv + lo.tr[db][1] + c16 * 16 * D * 2);
+        const vec8 vf = lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * DL * 2, lv + lo.tr[db][1] + c16 * 16 * DL * 2);
         o[db] = E::mfma32(vf, pf, o[db]);
       }
     }
@@ -209,6 +211,7 @@ void fwd_kernel(const KArgs a) {
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
+        if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
         const typename E::vec2 x0 = E::cvt2(o[db][4 * q4 + 0] * inv, o[db][4 * q4 + 1] * inv);
         const typename E::vec2 x1 = E::cvt2(o[db][4 * q4 + 2] * inv, o[db][4 * q4 + 3] * inv);
         typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
@@ -223,7 +226,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
   const int slots = (a.B * a.H + 7) / 8;
-  const size_t lds = 4 * BN * D * 2;
+  const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2;
   auto kern = fwd_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -247,6 +250,7 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
     case 128: return launch_cd<Tag, 128>(a, causal, doc, s);
     case 64: return launch_cd<Tag, 64>(a, causal, doc, s);
     case 32: return launch_cd<Tag, 32>(a, causal, doc, s);
+    case 16: return launch_cd<Tag, 16>(a, causal, doc, s);
     default: return -1;
   }
 }

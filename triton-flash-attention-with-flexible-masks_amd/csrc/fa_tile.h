@@ -119,7 +119,11 @@ FA_DEV void buf_load_lds16(buf_rsrc_t, char*, int, int) {}
 // (buffer_load_dwordx4 ... lds).  The per-lane byte offsets are computed once;
 // a tile is then addressed with one scalar offset, and rows past the end of the
 // matrix read as zero through the buffer's range check instead of being clamped.
-template <int D, int ROWS>
+// D is the row width of the LDS tile, GD (<= D) the width of the rows in memory; chunks past GD
+// are fetched from beyond the buffer's range, i.e. zero filled.
+constexpr int kOobOffset = (int)0x80000000;  // beyond any buffer this library accepts (< 2 GiB)
+
+template <int D, int ROWS, int GD = D>
 struct TileLoader {
   static constexpr int CPR = D / 8;      // 16-byte chunks per row
   static constexpr int RPI = 64 / CPR;   // rows per wave instruction
@@ -133,14 +137,14 @@ struct TileLoader {
   // base: first row of the (batch, head) slice; rs: row stride in elements
   FA_DEV void init(const void* base, int64_t rs, int nrows) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned bytes = (unsigned)((int64_t(nrows - 1) * rs + D) * 2);
+    const unsigned bytes = (unsigned)((int64_t(nrows - 1) * rs + GD) * 2);
     rsrc = make_rsrc(base, bytes);
     row_bytes = int(rs) * 2;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int row = (i * 4 + wave) * RPI + lane / CPR;
       const int c = (lane % CPR) ^ swz<D, SWZ_ROW>(row);
-      voff[i] = row * row_bytes + c * 16;
+      voff[i] = c < GD / 8 ? row * row_bytes + c * 16 : kOobOffset;
     }
   }
   // stream rows row0 .. row0+ROWS-1 into the tile at `lds`

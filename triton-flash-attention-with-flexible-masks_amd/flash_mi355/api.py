@@ -160,8 +160,10 @@ class FlashAttention(torch.autograd.Function):
                 p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
             delta = torch.empty_like(lse)
             dq = torch.empty_like(q, memory_format=torch.contiguous_format)
-            dk = torch.empty((B, H, N, D), dtype=k.dtype, device=q.device)
-            dv = torch.empty((B, H, N, D), dtype=v.dtype, device=q.device)
+            # the dk/dv kernel walks the query heads of a group itself and writes the group sum
+            # (the reference writes per query head and sums afterwards, flash_triton.py:594-595,635-637)
+            dk = torch.empty((B, Hk, N, D), dtype=k.dtype, device=q.device)
+            dv = torch.empty((B, Hk, N, D), dtype=v.dtype, device=q.device)
             p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
             p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
             _set4(p.o_stride, o); _set4(p.do_stride, do)
@@ -170,9 +172,6 @@ class FlashAttention(torch.autograd.Function):
             _cabi.check(L.fa_bwd_delta(ctypes.byref(p), stream), "fa_bwd_delta")
             _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
             _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
-            if num_groups > 1:  # flash_triton.py:635-637
-                dk = dk.reshape((B, Hk, num_groups, N, D)).sum(2, dtype=torch.float32).to(k.dtype)
-                dv = dv.reshape((B, Hk, num_groups, N, D)).sum(2, dtype=torch.float32).to(v.dtype)
         return dq, dk, dv, None, None, None, None, None
 
 
