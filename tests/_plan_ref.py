@@ -9,11 +9,11 @@ INT_MAX, INT_MIN = 2**31 - 1, -2**31
 
 def plan_q(eq, M):
     """eq: int array [M].  Returns perm [Pp], header dict, summaries list of dicts."""
-    Pp = (M + 127) // 128 * 128 + 128
+    Pp = (M + 255) // 256 * 256 + 256
     local = np.nonzero(eq < 0)[0]
     glob = np.nonzero(eq >= 0)[0]
     nL, nG = len(local), len(glob)
-    nLp = (nL + 127) // 128 * 128
+    nLp = (nL + 255) // 256 * 256
     perm = np.full(Pp, -1, np.int64)
     perm[:nL] = local
     perm[nLp:nLp + nG] = glob

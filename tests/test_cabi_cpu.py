@@ -82,8 +82,9 @@ def test_workspace_size():
     p.eq_stride[0], p.eq_stride[1], p.eq_stride[2] = 128, 0, 1       # ids shared by the heads
     p.ek_stride[0], p.ek_stride[1], p.ek_stride[2] = 4 * 256, 256, 1   # per head
     r256 = lambda x: (x + 255) // 256 * 256
-    Pp = 128 + 128
-    want = r256(128 * 4) + r256(4 * 256 * 4) + r256(Pp * 4) + r256(16) + r256(Pp // 64 * 32) + r256(4 * 4 * 32)
+    Pp = 256 + 256
+    want = (r256(128 * 4) + r256(4 * 256 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+            + r256(4 * 4 * 32))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want
 
 

@@ -176,19 +176,22 @@ def test_device_mask_plan_matches_host_restatement():
     torch.cuda.synchronize()
     ws = plan.workspace.cpu().numpy()
     r256 = lambda x: (x + 255) // 256 * 256
-    Mp, Np, Pp = (M + 63) // 64 * 64, (N + 63) // 64 * 64, (M + 127) // 128 * 128 + 128
+    Mp, Np, Pp = (M + 63) // 64 * 64, (N + 63) // 64 * 64, (M + 255) // 256 * 256 + 256
     nQs, nKs = Pp // 64, Np // 64
     off = 0
     take = lambda n: (off, off + n)
     o_eq = off; off += r256(B * H * Mp * 4)
     o_ek = off; off += r256(B * H * Np * 4)
     o_pm = off; off += r256(B * H * Pp * 4)
+    o_pq = off; off += r256(B * H * Pp * 4)
+    off += r256(B * H * ((Mp + 1023) // 1024) * 4)     # per-chunk counts of the partition
     o_hd = off; off += r256(B * H * 16)
     o_qs = off; off += r256(B * H * nQs * 32)
     o_ks = off; off += r256(B * H * nKs * 32)
     assert off == ws.size
     i32 = lambda o, n: ws[o:o + 4 * n].view(np.int32)
     perm = i32(o_pm, B * H * Pp).reshape(B, H, Pp)
+    peq = i32(o_pq, B * H * Pp).reshape(B, H, Pp)
     hdr = i32(o_hd, B * H * 4).reshape(B, H, 4)
     qs = i32(o_qs, B * H * nQs * 8).reshape(B, H, nQs, 8)
     ks = i32(o_ks, B * H * nKs * 8).reshape(B, H, nKs, 8)
@@ -198,6 +201,8 @@ def test_device_mask_plan_matches_host_restatement():
         for h in range(H):
             rp, rh, rq = P.plan_q(eq[b, h].astype(np.int64), M)
             assert np.array_equal(perm[b, h], rp)
+            assert np.array_equal(peq[b, h][rp >= 0], eq[b, h][rp[rp >= 0]])
+            rk = P.plan_k(ek[b, h].astype(np.int64), N)
             assert list(hdr[b, h]) == [rh["nL"], rh["nG"], rh["nLp"], rh["nT128"]]
             for t, s_ in enumerate(rq):
                 got = qs[b, h, t]
@@ -208,5 +213,11 @@ def test_device_mask_plan_matches_host_restatement():
                     assert (got[0], got[1]) == (s_["lo"], s_["hi"])
                 else:
                     assert got[0] > got[1]
+                # key-tile range of the plan: exactly the first / last tile the visit test admits
+                cand = [kt for kt, k_ in enumerate(rk) if P.visits(s_, k_, kt, True, N - M)]
+                if cand:
+                    assert (got[6], got[7]) == (cand[0], cand[-1])
+                else:
+                    assert got[7] < got[6]
             for t, s_ in enumerate(P.plan_k(ek[b, h].astype(np.int64), N)):
                 assert (ks[b, h, t, 0], ks[b, h, t, 1]) == (s_["lo"], s_["hi"])

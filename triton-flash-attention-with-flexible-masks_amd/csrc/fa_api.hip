@@ -96,7 +96,7 @@ static KArgs make_args(const fa_params* p) {
   a.gap = p->N > p->M ? p->N - p->M : 0;  // flash_triton.py:521
   a.scale = p->sm_scale;
   a.scale_log2e = p->sm_scale * kLog2e;
-  a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;
+  a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.peq = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;
   a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.pm_bs = a.pm_hs = a.qh_bs = a.qh_hs = 0;
   a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
   a.nQs = a.nKs = a.Pp = 0;
@@ -106,6 +106,7 @@ static KArgs make_args(const fa_params* p) {
     a.eq32 = reinterpret_cast<const int*>(ws + w.off_eq32);
     a.ek32 = reinterpret_cast<const int*>(ws + w.off_ek32);
     a.perm = reinterpret_cast<const int*>(ws + w.off_perm);
+    a.peq = reinterpret_cast<const int*>(ws + w.off_peq);
     a.qhdr = reinterpret_cast<const QHeader*>(ws + w.off_qhdr);
     a.qsum = reinterpret_cast<const IdSummary*>(ws + w.off_qsum);
     a.ksum = reinterpret_cast<const IdSummary*>(ws + w.off_ksum);

@@ -47,50 +47,79 @@ __global__ __launch_bounds__(256) void plan_k_kernel(const void* __restrict__ id
   if (lane == 0) {
     IdSummary s;
     s.lo = lo; s.hi = hi; s.glob = 0; s.rmin = tile * kSumRows; s.rmax = min(L, (tile + 1) * kSumRows) - 1;
-    s.nvalid = s.rmax - s.rmin + 1; s.pad0 = s.pad1 = 0;
+    s.nvalid = s.rmax - s.rmin + 1; s.kfirst = 0; s.klast = 0;
     sum[(int64_t(b) * H1 + h) * nS + tile] = s;
   }
 }
 
-// Query side: one workgroup per (batch, stored head).  Normalises the ids to int32,
-// builds the local-rows-first permutation with a stable two-way partition
-// (ballot + popcount prefix sums), then summarises every 64 entries of it.
-template <bool I64>
-__global__ __launch_bounds__(256) void plan_q_kernel(const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
-                                                     int M, int Mp, int Pp, int H1, int* __restrict__ eq32,
-                                                     int* __restrict__ perm, QHeader* __restrict__ hdr,
-                                                     IdSummary* __restrict__ qsum) {
-  __shared__ int sh_l[4], sh_g[4], sh_tot;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int64_t bh = int64_t(b) * H1 + h;
-  int* eqp = eq32 + bh * Mp;
-  int* pmp = perm + bh * Pp;
-  const int64_t base = b * s_b + h * s_h;
+// Query side, step 1: one workgroup per chunk of kPlanChunk rows.  Writes the int32 copy of the
+// ids, the number of local rows (eq < 0) of the chunk, and pre-fills the chunk's share of the
+// permuted order with -1.
+constexpr int kPlanChunk = 1024;
 
-  // pass 1: int32 copy of the ids and the number of local rows
-  int cnt = 0;
-  for (int r = tid; r < Mp; r += 256) {
-    const int v = r < M ? load_id<I64>(ids, base + int64_t(r) * s_r) : 0;
-    eqp[r] = v;
-    cnt += (r < M && v < 0) ? 1 : 0;
+template <bool I64>
+__global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
+                                                         int M, int Mp, int Pp, int nCh, int H1, int* __restrict__ eq32,
+                                                         int* __restrict__ perm, int* __restrict__ peq,
+                                                         int* __restrict__ cnt) {
+  __shared__ int sh[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int64_t bh = int64_t(b) * H1 + h;
+  const int64_t base = b * s_b + h * s_h;
+  int c = 0;
+#pragma unroll
+  for (int k = 0; k < kPlanChunk / 256; ++k) {
+    const int r = ch * kPlanChunk + k * 256 + tid;
+    if (r < Mp) {
+      const int v = r < M ? load_id<I64>(ids, base + int64_t(r) * s_r) : 0;
+      eq32[bh * Mp + r] = v;
+      c += (r < M && v < 0) ? 1 : 0;
+    }
+  }
+  // the last chunk also covers the tail of the permuted order (Pp > M)
+  const int p_end = ch == nCh - 1 ? Pp : min(Pp, (ch + 1) * kPlanChunk);
+  for (int i = ch * kPlanChunk + tid; i < p_end; i += 256) {
+    perm[bh * Pp + i] = -1;
+    peq[bh * Pp + i] = 0;
   }
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) cnt += __shfl_xor(cnt, off);
-  if (lane == 0) sh_l[wave] = cnt;
+  for (int off = 32; off >= 1; off >>= 1) c += __shfl_xor(c, off);
+  if (lane == 0) sh[wave] = c;
   __syncthreads();
-  const int nL = sh_l[0] + sh_l[1] + sh_l[2] + sh_l[3];
-  const int nG = M - nL;
-  const int nLp = (nL + 127) / 128 * 128;
-  __syncthreads();
+  if (tid == 0) cnt[bh * nCh + ch] = sh[0] + sh[1] + sh[2] + sh[3];
+}
 
-  // pass 2: stable partition, 256 rows per step
-  int baseL = 0, baseG = nLp;
+// Step 2: stable two-way partition.  Every chunk derives its output offsets from the counts of
+// the chunks before it, then places its rows with ballot / popcount prefix sums: local rows go to
+// perm[0 .. nL), global rows to perm[nLp .. nLp + nG), both in ascending row order.
+__global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp, int nCh, int H1,
+                                                           const int* __restrict__ eq32, const int* __restrict__ cnt,
+                                                           int* __restrict__ perm, int* __restrict__ peq,
+                                                           QHeader* __restrict__ hdr) {
+  __shared__ int sh_l[4], sh_g[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int64_t bh = int64_t(b) * H1 + h;
+  const int* eqp = eq32 + bh * Mp;
+  int* pmp = perm + bh * Pp;
+  int* pqp = peq + bh * Pp;
+  int before = 0, nL = 0;
+  for (int k = 0; k < nCh; ++k) {
+    const int c = cnt[bh * nCh + k];
+    before += k < ch ? c : 0;
+    nL += c;
+  }
+  const int nG = M - nL;
+  const int nLp = (nL + kPermAlign - 1) / kPermAlign * kPermAlign;
+  int baseL = before;
+  int baseG = nLp + (min(M, ch * kPlanChunk) - before);  // global rows before this chunk
   const unsigned long long lt = (1ull << lane) - 1ull;
-  for (int r0 = 0; r0 < M; r0 += 256) {
-    const int r = r0 + tid;
+#pragma unroll
+  for (int k = 0; k < kPlanChunk / 256; ++k) {
+    const int r = ch * kPlanChunk + k * 256 + tid;
     const bool valid = r < M;
-    const int v = valid ? eqp[r] : 0;  // written by this same thread in pass 1
+    const int v = valid ? eqp[r] : 0;
     const bool isL = valid && v < 0, isG = valid && v >= 0;
     const unsigned long long bl = __builtin_amdgcn_ballot_w64(isL), bg = __builtin_amdgcn_ballot_w64(isG);
     if (lane == 0) { sh_l[wave] = __builtin_popcountll(bl); sh_g[wave] = __builtin_popcountll(bg); }
@@ -102,68 +131,99 @@ __global__ __launch_bounds__(256) void plan_q_kernel(const void* __restrict__ id
       if (w < wave) { offL += cl; offG += cg; }
       totL += cl; totG += cg;
     }
-    if (isL) pmp[baseL + offL + __builtin_popcountll(bl & lt)] = r;
-    if (isG) pmp[baseG + offG + __builtin_popcountll(bg & lt)] = r;
+    if (isL) { const int pos = baseL + offL + __builtin_popcountll(bl & lt); pmp[pos] = r; pqp[pos] = v; }
+    if (isG) { const int pos = baseG + offG + __builtin_popcountll(bg & lt); pmp[pos] = r; pqp[pos] = v; }
     baseL += totL; baseG += totG;
     __syncthreads();
   }
-  for (int i = nL + tid; i < nLp; i += 256) pmp[i] = -1;
-  for (int i = nLp + nG + tid; i < Pp; i += 256) pmp[i] = -1;
-  __threadfence_block();
-  __syncthreads();
-
-  // pass 3: summaries of the permuted order, one wave per 64 entries
-  const int nT = Pp / kSumRows;
-  for (int t = wave; t < nT; t += 4) {
-    const int row = pmp[t * kSumRows + lane];
-    const bool valid = row >= 0;
-    const int v = valid ? eqp[row] : 0;
-    const bool local = valid && v < 0;
-    IdSummary s;
-    s.lo = wave_min(local ? v : 0x7fffffff);
-    s.hi = wave_max(local ? v : (int)0x80000000);
-    s.rmin = wave_min(valid ? row : 0x7fffffff);
-    s.rmax = wave_max(valid ? row : -1);
-    s.glob = __builtin_amdgcn_ballot_w64(valid && v >= 0) != 0 ? 1 : 0;
-    s.nvalid = __builtin_popcountll(__builtin_amdgcn_ballot_w64(valid));
-    s.pad0 = s.pad1 = 0;
-    if (lane == 0) qsum[bh * nT + t] = s;
-  }
-  if (tid == 0) {
+  if (ch == 0 && tid == 0) {
     QHeader q;
     q.nL = nL; q.nG = nG; q.nLp = nLp; q.nT128 = (nLp + (nG + 127) / 128 * 128) / 128;
     hdr[bh] = q;
   }
 }
 
+// Step 3: one wave per 64 entries of the permuted order: id / row-index summary, and the range
+// [kfirst, klast] of key tiles the entry's rows can need (by the key summaries and the causal
+// bound), so that the compute kernels start their tile search in the right place.
+__global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal_gap,
+                                                        const int* __restrict__ perm, const int* __restrict__ peq,
+                                                        const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= nQs) return;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int64_t bh = int64_t(b) * H1 + h;
+  const int row = perm[bh * Pp + t * kSumRows + lane];
+  const int v = peq[bh * Pp + t * kSumRows + lane];
+  const bool valid = row >= 0;
+  const bool local = valid && v < 0;
+  IdSummary s;
+  s.lo = wave_min(local ? v : 0x7fffffff);
+  s.hi = wave_max(local ? v : (int)0x80000000);
+  s.rmin = wave_min(valid ? row : 0x7fffffff);
+  s.rmax = wave_max(valid ? row : -1);
+  s.glob = __builtin_amdgcn_ballot_w64(valid && v >= 0) != 0 ? 1 : 0;
+  s.nvalid = __builtin_popcountll(__builtin_amdgcn_ballot_w64(valid));
+  int kfirst = 0x7fffffff, klast = -1;
+  if (H1 == HK1) {  // ids of both sides stored per the same heads: narrow the key range
+    const IdSummary* ks = ksum + bh * nKs;
+    const int kend = causal_gap >= 0 ? min(nKs, (causal_gap + s.rmax) / kSumRows + 1) : nKs;
+    for (int k0 = 0; k0 < kend; k0 += 64) {
+      const int k = k0 + lane;
+      bool cand = false;
+      if (k < kend) {
+        const IdSummary kk = ks[k];
+        cand = doc_may_keep(s.lo, s.hi, s.glob, kk.lo, kk.hi);
+      }
+      kfirst = min(kfirst, cand ? k : 0x7fffffff);
+      klast = max(klast, cand ? k : -1);
+    }
+    kfirst = wave_min(kfirst);
+    klast = wave_max(klast);
+  } else {
+    kfirst = 0; klast = nKs - 1;
+  }
+  s.kfirst = s.nvalid > 0 ? kfirst : 0x7fffffff;
+  s.klast = s.nvalid > 0 ? klast : -1;
+  if (lane == 0) qsum[bh * nQs + t] = s;
+}
+
 int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
   char* ws = reinterpret_cast<char*>(p->workspace);
   const bool i64 = p->id_dtype == FA_IDTYPE_I64;
+  int* eq32 = reinterpret_cast<int*>(ws + w.off_eq32);
+  int* ek32 = reinterpret_cast<int*>(ws + w.off_ek32);
+  int* perm = reinterpret_cast<int*>(ws + w.off_perm);
+  int* peq = reinterpret_cast<int*>(ws + w.off_peq);
+  int* cnt = reinterpret_cast<int*>(ws + w.off_cnt);
+  QHeader* hdr = reinterpret_cast<QHeader*>(ws + w.off_qhdr);
+  IdSummary* qsum = reinterpret_cast<IdSummary*>(ws + w.off_qsum);
+  IdSummary* ksum = reinterpret_cast<IdSummary*>(ws + w.off_ksum);
+  hipError_t e;
   {
-    int* out32 = reinterpret_cast<int*>(ws + w.off_ek32);
-    IdSummary* sum = reinterpret_cast<IdSummary*>(ws + w.off_ksum);
     const int64_t* st = p->ek_stride;
     dim3 grid((w.nKs + 3) / 4, w.Hk1, p->B);
     if (i64)
-      hipLaunchKernelGGL(plan_k_kernel<true>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, out32, sum);
+      hipLaunchKernelGGL(plan_k_kernel<true>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, ek32, ksum);
     else
-      hipLaunchKernelGGL(plan_k_kernel<false>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, out32, sum);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return (int)e;
+      hipLaunchKernelGGL(plan_k_kernel<false>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, ek32, ksum);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   {
-    int* eq32 = reinterpret_cast<int*>(ws + w.off_eq32);
-    int* perm = reinterpret_cast<int*>(ws + w.off_perm);
-    QHeader* hdr = reinterpret_cast<QHeader*>(ws + w.off_qhdr);
-    IdSummary* sum = reinterpret_cast<IdSummary*>(ws + w.off_qsum);
     const int64_t* st = p->eq_stride;
-    dim3 grid(w.Hq1, p->B);
+    dim3 grid(w.nCh, w.Hq1, p->B);
     if (i64)
-      hipLaunchKernelGGL(plan_q_kernel<true>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.Hq1, eq32, perm, hdr, sum);
+      hipLaunchKernelGGL(plan_count_kernel<true>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, cnt);
     else
-      hipLaunchKernelGGL(plan_q_kernel<false>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.Hq1, eq32, perm, hdr, sum);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return (int)e;
+      hipLaunchKernelGGL(plan_count_kernel<false>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, cnt);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(plan_scatter_kernel, grid, dim3(256), 0, s, p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, cnt, perm, peq, hdr);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+    const int gap = p->N > p->M ? p->N - p->M : 0;
+    hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
+                       p->causal ? gap : -1, perm, peq, ksum, qsum);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   return 0;
 }

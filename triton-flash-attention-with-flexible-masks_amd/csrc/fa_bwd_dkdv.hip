@@ -45,7 +45,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   // turn with K/V staying in registers, so dK/dV leave the kernel already summed over the group
   const int nKt = (a.N + BK - 1) / BK;
   int kt, bhk;
-  if (!block_to_tile(nKt, a.B * a.Hk, kt, bhk)) return;  // causal: the first key tiles see the most rows
+  if (!block_to_tile(nKt, a.B * a.Hk, false, kt, bhk)) return;  // causal: the first key tiles see the most rows
   const int b = bhk / a.Hk, hk = bhk % a.Hk;
 
   const T* kp = reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs;
@@ -109,8 +109,8 @@ void bwd_dkdv_kernel(const KArgs a) {
       ldQ.issue(m0, smem + bufi * TILE_BYTES);
       ldO.issue(m0, smem + (2 + bufi) * TILE_BYTES);
       const int r = m0 + lane < a.M ? m0 + lane : a.M - 1;
-      if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
-      if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
+      if (wave == 0) glb_load_lds4(lsep + r, aux);
+      if (wave == 1) glb_load_lds4(delp + r, aux + 256);
     } else {
 #pragma unroll
       for (int i = 0; i < Loader::PER; ++i) {
@@ -119,10 +119,10 @@ void bwd_dkdv_kernel(const KArgs a) {
         buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * 4 + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
       }
       const int r = ri_aux >= 0 ? ri_aux : 0;
-      if (wave == 0) __builtin_amdgcn_global_load_lds(FA_GLB(lsep + r), FA_LDS(aux), 4, 0, 0);
-      if (wave == 1) __builtin_amdgcn_global_load_lds(FA_GLB(delp + r), FA_LDS(aux + 256), 4, 0, 0);
-      if (wave == 2) __builtin_amdgcn_global_load_lds(FA_GLB(eqp + r), FA_LDS(aux + 512), 4, 0, 0);
-      if (wave == 3) __builtin_amdgcn_global_load_lds(FA_GLB(pmp + tile * BQ + lane), FA_LDS(aux + 768), 4, 0, 0);
+      if (wave == 0) glb_load_lds4(lsep + r, aux);
+      if (wave == 1) glb_load_lds4(delp + r, aux + 256);
+      if (wave == 2) glb_load_lds4(eqp + r, aux + 512);
+      if (wave == 3) glb_load_lds4(pmp + tile * BQ + lane, aux + 768);
     }
   };
 
@@ -158,29 +158,40 @@ void bwd_dkdv_kernel(const KArgs a) {
         const vec8 da = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * DL * 2);
         dp = E::mfma32(da, vf[ks], dp);
       }
-      // s -> P, dp -> dS for this lane's 16 query rows of the block
+      // s -> P for this lane's 16 query rows of the block
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
         const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
-        const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
-        i32x4 eqv = {0, 0, 0, 0};
-        i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
-        if (DOC && need_mask) {
-          eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
-          rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
-        }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float p = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
-          if (need_mask) {
+        for (int t = 0; t < 4; ++t) s[4 * q4 + t] = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
+      }
+      if (need_mask) {
+        asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int i0 = 32 * qb + 8 * q4 + 4 * g;
+          i32x4 eqv = {0, 0, 0, 0};
+          i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
+          if (DOC) {
+            eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+            rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+          }
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
             const int i = rowv[t];
             const bool keep = (i >= 0) && (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
-            p = keep ? p : 0.f;
+            s[4 * q4 + t] = keep ? s[4 * q4 + t] : 0.f;
           }
-          s[4 * q4 + t] = p;
-          dp[4 * q4 + t] = p * (dp[4 * q4 + t] - dl[t]);
         }
+      }
+      // dp -> dS = P * (dP - delta)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dp[4 * q4 + t] = s[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
       }
 #pragma unroll
       for (int half = 0; half < 2; ++half) {

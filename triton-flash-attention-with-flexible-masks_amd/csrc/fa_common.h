@@ -38,6 +38,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // Rows covered by one entry of the id summaries written by the mask plan.
 constexpr int kSumRows = 64;
+// The local-row part of the permuted order is padded to this many entries, so that a
+// workgroup of up to 256 query rows never mixes local and global rows.
+constexpr int kPermAlign = 256;
 
 struct bf16_t {};
 struct fp16_t {};
@@ -127,7 +130,7 @@ FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j) {
 // into LOCAL rows (eq < 0: see only keys with the same id) and GLOBAL rows
 // (eq >= 0: see every key), each group kept in ascending row order:
 //   perm[0 .. nL)            local rows            (padded with -1 up to nLp,
-//   perm[nLp .. nLp + nG)    global rows            nLp = nL rounded up to 128)
+//   perm[nLp .. nLp + nG)    global rows            nLp = nL rounded up to kPermAlign)
 // Query-side tiles are tiles of this permuted order, so a tile is either all
 // local (it only needs the key tiles whose id interval meets its own) or all
 // global (no doc test at all, plain causal structure).  Keys stay in natural
@@ -138,7 +141,7 @@ struct IdSummary {
   int glob;        // query side: 1 if the tile holds global rows
   int rmin, rmax;  // query side: smallest / largest original row index of the tile (rmax = -1 if empty)
   int nvalid;      // query side: rows of the tile that exist
-  int pad0, pad1;
+  int kfirst, klast;  // query side: first / last key tile (of 64 keys) the rows can need (klast < kfirst: none)
 };
 
 struct QHeader {
@@ -171,6 +174,7 @@ struct KArgs {
   const int* eq32;        // [B, Hq', Mp]   ids in natural row order
   const int* ek32;        // [B, Hk', Np]
   const int* perm;        // [B, Hq', Pp]   permuted order -> original row (or -1)
+  const int* peq;         // [B, Hq', Pp]   id of that row
   const QHeader* qhdr;    // [B, Hq']
   const IdSummary* qsum;  // [B, Hq', nQs]  per 64 entries of the permuted order
   const IdSummary* ksum;  // [B, Hk', nKs]  per 64 keys
@@ -201,7 +205,8 @@ struct WsLayout {
   int Mp, Np;             // M, N rounded up to kSumRows
   int Pp;                 // length of the permuted order
   int nQs, nKs;
-  uint64_t off_eq32, off_ek32, off_perm, off_qhdr, off_qsum, off_ksum, total;  // bytes
+  int nCh;                // row chunks of the partition kernels
+  uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum, total;  // bytes
 };
 
 inline WsLayout ws_layout(const fa_params* p) {
@@ -211,13 +216,16 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.Mp = (p->M + kSumRows - 1) / kSumRows * kSumRows;
   w.nKs = (p->N + kSumRows - 1) / kSumRows;
   w.Np = w.nKs * kSumRows;
-  w.Pp = (p->M + 127) / 128 * 128 + 128;
+  w.Pp = (p->M + kPermAlign - 1) / kPermAlign * kPermAlign + kPermAlign;
   w.nQs = w.Pp / kSumRows;
   uint64_t o = 0;
   auto take = [&](uint64_t bytes) { uint64_t r = o; o += (bytes + 255) & ~uint64_t(255); return r; };
   w.off_eq32 = take(uint64_t(p->B) * w.Hq1 * w.Mp * 4);
   w.off_ek32 = take(uint64_t(p->B) * w.Hk1 * w.Np * 4);
   w.off_perm = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
+  w.off_peq = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
+  w.nCh = (w.Mp + 1023) / 1024;
+  w.off_cnt = take(uint64_t(p->B) * w.Hq1 * w.nCh * 4);
   w.off_qhdr = take(uint64_t(p->B) * w.Hq1 * sizeof(QHeader));
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));

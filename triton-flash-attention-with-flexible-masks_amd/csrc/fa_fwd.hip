@@ -44,10 +44,10 @@ void fwd_kernel(const KArgs a) {
   // order and see the longest key ranges; without ids the last rows do
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
   int slot, bh;
-  if (!block_to_tile(nQt, a.B * a.H, slot, bh)) return;
+  if (!block_to_tile(nQt, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
   QTileCtx<CAUSAL, DOC> qc;
-  if (!qc.init(a, b, h, nQt - 1 - slot)) return;
+  if (!qc.init(a, b, h, nQt - 1 - slot, threadIdx.x >> 6)) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
 
@@ -70,7 +70,7 @@ void fwd_kernel(const KArgs a) {
   }
 
   TileIter it;
-  it.init_keys(0, (qc.hi_key(a) + BN - 1) / BN, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+  it.init_keys(qc.first_tile(), qc.last_tile(a), qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
@@ -108,6 +108,7 @@ void fwd_kernel(const KArgs a) {
       }
     }
     if (need_mask) {
+      asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll

@@ -29,91 +29,45 @@ FA_DEV int swz(int row) {
   return 0;
 }
 
-// Asynchronously copy ROWS x D elements (rows row0 .. row0+ROWS-1 of a [*, D]
-// matrix with row stride `rs` elements, rows clamped to nrows-1) from global
-// memory straight into LDS, all 256 threads cooperating.  Completion is
-// observed with s_waitcnt vmcnt(0) followed by a workgroup barrier.
-template <typename T, int D, int ROWS, int SWZ>
-FA_DEV void tile_load_async(const T* __restrict__ g, int64_t rs, int row0, int nrows, char* lds) {
-  constexpr int CPR = D / 8;          // chunks per row
-  constexpr int RPI = 64 / CPR;       // rows per wave instruction
-  constexpr int NI = ROWS / RPI;      // wave instructions per tile
-  static_assert(NI % 4 == 0, "tile must split evenly over 4 waves");
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < NI / 4; ++i) {
-    const int inst = i * 4 + wave;
-    const int row = inst * RPI + lane / CPR;
-    const int pc = lane % CPR;
-    const int c = pc ^ swz<D, SWZ>(row);
-    int grow = row0 + row;
-    grow = grow < nrows ? grow : nrows - 1;
-    const T* src = g + int64_t(grow) * rs + c * 8;
-    __builtin_amdgcn_global_load_lds(FA_GLB(src), FA_LDS(lds + inst * 1024), 16, 0, 0);
-  }
+// ---------------------------------------------------------------------------
+// Asynchronous global -> LDS copies (the data never passes through registers).
+// They are issued from inline assembly on purpose: written with the compiler's
+// builtins, every later LDS read is preceded by s_waitcnt vmcnt(0), because the
+// compiler cannot tell that the tile being filled is not the tile being read, and
+// the copy of the next tile then no longer overlaps the arithmetic on this one.
+// Completion is observed explicitly: wait_async_loads() followed by a workgroup
+// barrier, before the first read of the tile.
+// ---------------------------------------------------------------------------
+// Raw buffer resource (stride 0): base address, byte range, gfx9 data-format word.
+typedef i32x4 buf_rsrc_t;
+
+FA_DEV buf_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+  // wave-uniform by construction; readfirstlane tells the compiler so (the words must sit in SGPRs)
+  buf_rsrc_t r = {__builtin_amdgcn_readfirstlane((int)(unsigned)p), __builtin_amdgcn_readfirstlane((int)((p >> 32) & 0xffff)),
+                  __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+  return r;
 }
 
-// Same, with an explicit list of row indices (gathered rows), idx[r] already clamped.
-template <typename T, int D, int ROWS, int SWZ>
-FA_DEV void tile_load_async_rows(const T* __restrict__ g, int64_t rs, const int* __restrict__ idx, char* lds) {
-  constexpr int CPR = D / 8;
-  constexpr int RPI = 64 / CPR;
-  constexpr int NI = ROWS / RPI;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < NI / 4; ++i) {
-    const int inst = i * 4 + wave;
-    const int row = inst * RPI + lane / CPR;
-    const int pc = lane % CPR;
-    const int c = pc ^ swz<D, SWZ>(row);
-    const T* src = g + int64_t(idx[row]) * rs + c * 8;
-    __builtin_amdgcn_global_load_lds(FA_GLB(src), FA_LDS(lds + inst * 1024), 16, 0, 0);
-  }
+// LDS byte address of a pointer into the workgroup's dynamic shared memory
+FA_DEV unsigned lds_addr(const char* p) {
+  return (unsigned)(unsigned long long)(p);  // the low 32 bits of a generic LDS address are the LDS offset
+}
+
+// 16 bytes per lane from base + voff + soff into lds + 16 * lane (out of range reads give 0)
+FA_DEV void buf_load_lds16(buf_rsrc_t r, const char* lds, int voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_addr(lds))), "v"(voff), "s"(r), "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+
+// 4 bytes per lane from the lane's own address into lds + 4 * lane
+FA_DEV void glb_load_lds4(const void* src, const char* lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_addr(lds))), "v"(src) : "memory", "m0");
 }
 
 FA_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-// 8 consecutive elements of row `row` starting at element 8*chunk (A or B operand).
-template <typename E, int D, int SWZ>
-FA_DEV typename E::vec8 frag_row(const char* lds, int row, int chunk) {
-  const int pc = chunk ^ swz<D, SWZ>(row);
-  return *reinterpret_cast<const typename E::vec8*>(lds + row * (D * 2) + pc * 16);
-}
-
-// Transposed operand: for the 16 rows rbase .. rbase+15 of the tile and the 32
-// columns 32*db .. 32*db+31, returns for lane l (col = 32*db + (l & 31), g = l >> 5)
-// the 8 values of rows rbase + {4g..4g+3, 8+4g..8+4g+3} at that column, which is the
-// k-slot order of an accumulator block reused as the other MFMA operand.
-template <typename E, int D, int SWZ>
-FA_DEV typename E::vec8 frag_tr(const char* lds, int rbase, int db) {
-  const int l = threadIdx.x & 63;
-  const int i = l & 15, e = i >> 2, c4 = i & 3, hd = (l >> 4) & 1, g = l >> 5;
-  const int chunk = 4 * db + 2 * hd + (c4 >> 1);
-  const int sub = (c4 & 1) * 8;
-  const int r0 = rbase + 4 * g + e;
-  const int r1 = r0 + 8;
-  typename E::vec4 lo = E::lds_tr(lds + r0 * (D * 2) + ((chunk ^ swz<D, SWZ>(r0)) * 16) + sub);
-  typename E::vec4 hi = E::lds_tr(lds + r1 * (D * 2) + ((chunk ^ swz<D, SWZ>(r1)) * 16) + sub);
-  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// Buffer resource and buffer -> LDS load.  The resource type and the builtins exist
-// only in the device pass; the host pass (which still parses the kernels to emit
-// their launch stubs) sees a plain struct and empty bodies.
-#if defined(__HIP_DEVICE_COMPILE__)
-typedef __amdgpu_buffer_rsrc_t buf_rsrc_t;
-FA_DEV buf_rsrc_t make_rsrc(const void* base, unsigned bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-// 16 bytes per lane from base + voff + soff into lds + 16 * lane
-FA_DEV void buf_load_lds16(buf_rsrc_t r, char* lds, int voff, int soff) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, FA_LDS(lds), 16, voff, soff, 0, 0);
-}
-#else
-struct buf_rsrc_t { int w[4]; };
-FA_DEV buf_rsrc_t make_rsrc(const void*, unsigned) { return buf_rsrc_t(); }
-FA_DEV void buf_load_lds16(buf_rsrc_t, char*, int, int) {}
-#endif
 
 // Global -> LDS tile streamer built on buffer loads with the LDS destination
 // (buffer_load_dwordx4 ... lds).  The per-lane byte offsets are computed once;
@@ -123,13 +77,12 @@ FA_DEV void buf_load_lds16(buf_rsrc_t, char*, int, int) {}
 // are fetched from beyond the buffer's range, i.e. zero filled.
 constexpr int kOobOffset = (int)0x80000000;  // beyond any buffer this library accepts (< 2 GiB)
 
-template <int D, int ROWS, int GD = D>
+template <int D, int ROWS, int GD = D, int NW = 4>
 struct TileLoader {
   static constexpr int CPR = D / 8;      // 16-byte chunks per row
   static constexpr int RPI = 64 / CPR;   // rows per wave instruction
   static constexpr int NI = ROWS / RPI;  // wave instructions per tile
-  static constexpr int PER = NI / 4;     // per wave
-  static_assert(NI % 4 == 0, "tile must split evenly over 4 waves");
+  static constexpr int PER = (NI + NW - 1) / NW;  // per wave (NW waves share the tile)
   buf_rsrc_t rsrc;
   int voff[PER];
   int row_bytes;
@@ -142,7 +95,7 @@ struct TileLoader {
     row_bytes = int(rs) * 2;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int row = (i * 4 + wave) * RPI + lane / CPR;
+      const int row = (i * NW + wave) * RPI + lane / CPR;
       const int c = (lane % CPR) ^ swz<D, SWZ_ROW>(row);
       voff[i] = c < GD / 8 ? row * row_bytes + c * 16 : kOobOffset;
     }
@@ -153,7 +106,7 @@ struct TileLoader {
     const int soff = row0 * row_bytes;
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-      buf_load_lds16(rsrc, lds + (i * 4 + wave) * 1024, voff[i], soff);
+      if (NI % NW == 0 || i * NW + wave < NI) buf_load_lds16(rsrc, lds + (i * NW + wave) * 1024, voff[i], soff);
   }
 };
 
@@ -261,16 +214,19 @@ struct QTileCtx {
   int eq_i;
   int w_lo, w_hi, w_glob, w_rmin, w_rmax;  // this wave's 32 rows
   int g_lo, g_hi, g_glob, g_rmax;          // the workgroup's 128 rows
+  int g_kfirst, g_klast;                   // key tiles (of 64) those rows can need, from the mask plan
   const int* ekp;
   const IdSummary* ksum;
 
   // tile: index of the 128-row tile (natural order, or permuted order with ids).
   // Returns false when the tile holds no row.
-  FA_DEV bool init(const KArgs& a, int b, int h, int tile) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // wave: index (0..3) of this wave inside the 128-row tile.
+  FA_DEV bool init(const KArgs& a, int b, int h, int tile, int wave) {
+    const int lane = threadIdx.x & 63;
     const int lq = lane & 31;
     eq_i = 0; ekp = nullptr; ksum = nullptr;
     w_lo = 0; w_hi = -1; w_glob = 1; g_lo = 0; g_hi = -1; g_glob = 1;
+    g_kfirst = 0; g_klast = 0x3fffffff;
     if (!DOC) {
       const int m0 = tile * 128, mw = m0 + wave * 32;
       row = mw + lq < a.M ? mw + lq : -1;
@@ -278,16 +234,21 @@ struct QTileCtx {
       if (w_rmax < w_rmin) w_rmax = -1;
       g_rmax = min(m0 + 127, a.M - 1);
     } else {
-      const QHeader hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
-      if (tile >= hd.nT128) return false;
-      row = a.perm[b * a.pm_bs + h * a.pm_hs + tile * 128 + wave * 32 + lq];
-      const IdSummary* qs = a.qsum + b * a.qs_bs + h * a.qs_hs + 2 * tile;
-      const IdSummary s0 = qs[0], s1 = qs[1];
-      g_lo = min(s0.lo, s1.lo); g_hi = max(s0.hi, s1.hi); g_glob = s0.glob | s1.glob;
-      g_rmax = max(s0.rmax, s1.rmax);
       ekp = a.ek32 + b * a.ek_bs + h * a.ek_hs;
       ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
-      eq_i = row >= 0 ? a.eq32[b * a.eq_bs + h * a.eq_hs + row] : 0;
+      const IdSummary* qs = a.qsum + b * a.qs_bs + h * a.qs_hs + 2 * tile;
+      const IdSummary s0 = qs[0], s1 = qs[1];
+      const int64_t pos = b * a.pm_bs + h * a.pm_hs + tile * 128 + wave * 32 + lq;
+      row = a.perm[pos];     // issued together with the summaries: no dependent load chain
+      eq_i = a.peq[pos];
+      if (s0.nvalid + s1.nvalid == 0) {  // no rows: every decision below says "skip"
+        row = -1; rowc = 0; eq_i = 0; w_rmin = 0x7fffffff; w_rmax = -1; w_glob = 0;
+        g_lo = 0x7fffffff; g_hi = (int)0x80000000; g_glob = 0; g_rmax = -1;
+        return false;
+      }
+      g_lo = min(s0.lo, s1.lo); g_hi = max(s0.hi, s1.hi); g_glob = s0.glob | s1.glob;
+      g_rmax = max(s0.rmax, s1.rmax);
+      g_kfirst = min(s0.kfirst, s1.kfirst); g_klast = max(s0.klast, s1.klast);
       const bool local = (eq_i < 0) && (row >= 0);
       int lo = local ? eq_i : 0x7fffffff, hi = local ? eq_i : (int)0x80000000;
       int rmin = row >= 0 ? row : 0x7fffffff, rmax = row;
@@ -304,8 +265,12 @@ struct QTileCtx {
     rowc = row >= 0 ? row : 0;
     return true;
   }
-  // one past the last key any row of the workgroup can see
-  FA_DEV int hi_key(const KArgs& a) const { return CAUSAL ? min(a.N, a.gap + g_rmax + 1) : a.N; }
+  // range [first, last) of 64-key tiles the workgroup has to look at
+  FA_DEV int first_tile() const { return g_kfirst < 0x3fffffff ? g_kfirst : 0; }
+  FA_DEV int last_tile(const KArgs& a) const {
+    const int hi_key = CAUSAL ? min(a.N, a.gap + g_rmax + 1) : a.N;
+    return min((hi_key + 63) / 64, g_klast + 1);
+  }
 
   // wave-level decisions for key tile `cur` (keys n0 .. n0+BN-1)
   FA_DEV void decide(const KArgs& a, int cur, int n0, int BN, bool& skip, bool& need_mask) const {
@@ -319,13 +284,25 @@ struct QTileCtx {
   }
 };
 
-// blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head):
-// consecutive workgroup ids land on different XCDs, so every XCD is given whole
-// heads (its L2 then keeps that head's K/V or Q/dO).  Returns false for padding ids.
-FA_DEV bool block_to_tile(int ntile, int BH, int& tile_slot, int& bh) {
+// blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head).
+// Consecutive workgroup ids land on different XCDs, so every XCD is given whole
+// heads (its L2 then keeps that head's K/V or Q/dO).  Inside an XCD the order is
+//   head-major (tile_major = false): one head after the other -- best L2 reuse when
+//        every tile streams most of the head (no ids);
+//   tile-major (tile_major = true): tile slot 0 of all the XCD's heads, then slot 1, ...
+//        -- with ids the few heavy tiles (global rows) of EVERY head start at once
+//        instead of queueing behind the light tiles of the heads before them.
+// Returns false for padding ids.
+FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, int& bh) {
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  bh = (idx / ntile) * 8 + xcd;
-  tile_slot = idx % ntile;
+  const int heads = (BH + 7) / 8;  // heads per XCD
+  if (tile_major) {
+    bh = (idx % heads) * 8 + xcd;
+    tile_slot = idx / heads;
+  } else {
+    bh = (idx / ntile) * 8 + xcd;
+    tile_slot = idx % ntile;
+  }
   return bh < BH;
 }
 
