@@ -1,30 +1,31 @@
-// dK/dV kernel of the split backward: 128 keys per workgroup (32 per wave) held
-// in registers, query-side tiles (Q, dO, LSE, delta, eq, row index) streamed
-// through LDS.  Replaces _bwd_kv_kernel of the reference (flash_triton.py:175-321).
+// dK/dV kernel of the split backward.  Replaces _bwd_kv_kernel of the reference
+// (flash_triton.py:175-321).
 //
-//   S    = Q K^T           A = Q rows (LDS),  B = K^T (registers, whole kernel)
-//   dP   = dO V^T          A = dO rows (LDS), B = V^T (registers, whole kernel)
-//   P    = exp2(S*c - L), masked elements -> 0           (flash_triton.py:269-280)
-//   dS   = P * (dP - delta)                              (flash_triton.py:301)
-//   dV^T += dO^T P         A = dO^T via ds_read_b64_tr_b16, B = P from the accumulators
-//   dK^T += Q^T dS         A = Q^T  via ds_read_b64_tr_b16, B = dS
-//   dK   = dK * sm_scale                                 (flash_triton.py:313)
-// In the accumulator layout each lane owns ONE key column and 16 query rows of
-// every 32-row block, so LSE / delta / eq / row index are read as broadcast
-// 16-byte LDS loads.
-// With document ids the query side is walked in the permuted (local rows first)
-// order of the mask plan: tiles are gathered row by row through the permutation,
-// and only tiles whose id interval and row range can meet this workgroup's keys
-// are visited.
-// The query heads of a grouped-query group are walked inside the kernel, so dK, dV are
-// written once, already summed (the reference sums afterwards, flash_triton.py:635-637).
-
+// One workgroup = 128 keys, 8 waves.  The two waves that share a SIMD own the SAME 32 keys and
+// split the work by role, so that each needs only one operand fragment set and one accumulator
+// set (two waves per SIMD fit in the register file, and one role's vector work overlaps the
+// other role's matrix work):
+//   role 0 ("score" wave)                       role 1 ("gradient" wave)
+//   S  = Q K^T      A = Q rows, B = K^T (regs)  dP = dO V^T     A = dO rows, B = V^T (regs)
+//   P  = exp2(S*c - L), masked -> 0             ---------------- barrier ----------------
+//   P (fp32) -> LDS                             dS = P * (dP - delta)      (P read from LDS)
+//   dV^T += dO^T P  A = dO^T (transposed read)  dK^T += Q^T dS  A = Q^T (transposed read)
+// (flash_triton.py:265-308; dK is scaled by sm_scale at the end, :313).  In the accumulator
+// layout each lane owns ONE key column and 16 query rows of every 32-row block, so LSE / delta /
+// eq / row index are read as broadcast 16-byte LDS loads, and P travels between the two roles in
+// exactly the register layout both of them use.
+// Query-side tiles (Q, dO, LSE, delta, eq, row index; 64 rows) are streamed through LDS, two
+// buffers.  With document ids the query side is walked in the permuted (local rows first) order
+// of the mask plan: tiles are gathered row by row through the permutation (row indices fetched
+// one tile ahead), and only tiles whose id interval and row range can meet this workgroup's keys
+// are visited.  The query heads of a grouped-query group are walked inside the kernel, so dK, dV
+// are written once, already summed (the reference sums afterwards, flash_triton.py:635-637).
 #include "fa_tile.h"
 
 namespace fa {
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
@@ -33,38 +34,35 @@ void bwd_dkdv_kernel(const KArgs a) {
   constexpr int DL = D < 32 ? 32 : D;  // LDS row width: D = 16 is staged as 32 columns, the upper 16 zero
   constexpr int DBN = DL / 32;
   constexpr int TILE_BYTES = BQ * DL * 2;
-  constexpr int AUX_OFF = 4 * TILE_BYTES;  // [2 buffers][4 arrays][64] x 4 bytes
+  constexpr int AUX_OFF = 4 * TILE_BYTES;      // [2 buffers][4 arrays][64] x 4 bytes
   constexpr int AUX_BYTES = 1024;
-  using Loader = TileLoader<DL, BQ, D>;
+  constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][4 key blocks][4 x 1024] fp32 P
+  constexpr int P_BYTES = 4096;
+  using Loader = TileLoader<DL, BQ, D, 8>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int role = wave >> 2, kb = wave & 3;
   const int lq = lane & 31, g = lane >> 5;
 
-  // one workgroup per (key tile, batch, kv head); the query heads of the group are walked in
-  // turn with K/V staying in registers, so dK/dV leave the kernel already summed over the group
+  // one workgroup per (key tile, batch, kv head)
   const int nKt = (a.N + BK - 1) / BK;
   int kt, bhk;
   if (!block_to_tile(nKt, a.B * a.Hk, false, kt, bhk)) return;  // causal: the first key tiles see the most rows
   const int b = bhk / a.Hk, hk = bhk % a.Hk;
 
-  const T* kp = reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs;
-  const T* vp = reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs;
-  T* dkp = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs;
-  T* dvp = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs;
-
   const int n0 = kt * BK;
-  const int nw = n0 + wave * 32;
+  const int nw = n0 + kb * 32;
   const int key = nw + lq;
   const int keyc = key < a.N ? key : a.N - 1;
 
-  // K^T, V^T fragments (B operands): lane holds d = 16*ks + 8*g .. +7 of its key row.
-  vec8 kf[KS], vf[KS];
+  // B operand held for the whole kernel: K^T for the score wave, V^T for the gradient wave.
+  // Lane holds d = 16*ks + 8*g .. +7 of its key row.
+  const T* srcp = role == 0 ? reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs + int64_t(keyc) * a.k_rs
+                            : reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs + int64_t(keyc) * a.v_rs;
+  vec8 frag[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    kf[ks] = *reinterpret_cast<const vec8*>(kp + int64_t(keyc) * a.k_rs + ks * 16 + g * 8);
-    vf[ks] = *reinterpret_cast<const vec8*>(vp + int64_t(keyc) * a.v_rs + ks * 16 + g * 8);
-  }
+  for (int ks = 0; ks < KS; ++ks) frag[ks] = *reinterpret_cast<const vec8*>(srcp + ks * 16 + g * 8);
   const float c = a.scale_log2e;
 
   // per query head state (set at the top of the head loop)
@@ -83,16 +81,17 @@ void bwd_dkdv_kernel(const KArgs a) {
   int g_coff[Loader::PER], g_rit[Loader::PER];
 #pragma unroll
   for (int i = 0; i < Loader::PER; ++i) {
-    g_rit[i] = (i * 4 + wave) * Loader::RPI + lane / Loader::CPR;
+    g_rit[i] = ((i * 8 + wave) * Loader::RPI + lane / Loader::CPR) % BQ;
     const int gc = (lane % Loader::CPR) ^ swz<DL, SWZ_ROW>(g_rit[i]);
     g_coff[i] = gc < D / 8 ? gc * 16 : kOobOffset;
   }
 
-  f32x16 dk[DBN], dv[DBN];
+  // dV^T (score wave) or dK^T (gradient wave): lane = key column, registers = d rows
+  f32x16 acc[DBN];
 #pragma unroll
   for (int db = 0; db < DBN; ++db)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 
   // row indices of a permuted tile this lane needs: PER tile rows for Q/dO, one for the aux arrays
   int ri_t[Loader::PER] = {};
@@ -103,7 +102,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     ri_aux = pmp[tile * BQ + lane];
   };
   auto load_tile = [&](int tile, int bufi) {
-    char* aux = smem + AUX_OFF + bufi * AUX_BYTES;
+    const char* aux = smem + AUX_OFF + bufi * AUX_BYTES;
     if (!DOC) {
       const int m0 = tile * BQ;
       ldQ.issue(m0, smem + bufi * TILE_BYTES);
@@ -114,9 +113,11 @@ void bwd_dkdv_kernel(const KArgs a) {
     } else {
 #pragma unroll
       for (int i = 0; i < Loader::PER; ++i) {
-        const int r = ri_t[i] >= 0 ? ri_t[i] : 0;
-        buf_load_lds16(ldQ.rsrc, smem + bufi * TILE_BYTES + (i * 4 + wave) * 1024, r * ldQ.row_bytes + g_coff[i], 0);
-        buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * 4 + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
+        if (Loader::NI % 8 == 0 || i * 8 + wave < Loader::NI) {
+          const int r = ri_t[i] >= 0 ? ri_t[i] : 0;
+          buf_load_lds16(ldQ.rsrc, smem + bufi * TILE_BYTES + (i * 8 + wave) * 1024, r * ldQ.row_bytes + g_coff[i], 0);
+          buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * 8 + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
+        }
       }
       const int r = ri_aux >= 0 ? ri_aux : 0;
       if (wave == 0) glb_load_lds4(lsep + r, aux);
@@ -126,13 +127,18 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
 
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // One query tile.  BUF is a compile-time constant so every LDS address is base + immediate.
   auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
     const char* lqt = smem + BUF * TILE_BYTES;
     const char* ldo = smem + (2 + BUF) * TILE_BYTES;
     const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
+    const char* t1 = role == 0 ? lqt : ldo;   // rows operand of the first product
+    const char* t2 = role == 0 ? ldo : lqt;   // transposed operand of the second product
     const int m0 = cur * BQ;  // natural order only
 
-    // wave-level decisions: the tile's 64 rows against keys nw..nw+31
+    // wave-level decisions (identical for the two waves of a pair): the tile's 64 rows against keys nw..nw+31
     bool skip, need_mask;
     if (!DOC) {
       skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
@@ -143,76 +149,81 @@ void bwd_dkdv_kernel(const KArgs a) {
       need_mask = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31)) ||
                   !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
     }
-    if (skip) return;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      f32x16 s = zero, dp = zero;
+      char* pbuf = smem + P_OFF + (qb * 4 + kb) * P_BYTES + lane * 16;
+      f32x16 x = zero;
+      if (!skip) {
+        // first product: S (score wave) or dP (gradient wave)
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const vec8 qa = lds_row8<E>(lqt + lo.row[ks] + qb * 32 * DL * 2);
-        s = E::mfma32(qa, kf[ks], s);
-      }
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec8 ra = lds_row8<E>(t1 + lo.row[ks] + qb * 32 * DL * 2);
+          x = E::mfma32(ra, frag[ks], x);
+        }
+        if (role == 0) {
+          // S -> P for this lane's 16 query rows of the block
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const vec8 da = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * DL * 2);
-        dp = E::mfma32(da, vf[ks], dp);
-      }
-      // s -> P for this lane's 16 query rows of the block
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
+            const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
-        const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) s[4 * q4 + t] = fast_exp2(__builtin_fmaf(s[4 * q4 + t], c, -Lv[t]));
-      }
-      if (need_mask) {
-        asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int i0 = 32 * qb + 8 * q4 + 4 * g;
-          i32x4 eqv = {0, 0, 0, 0};
-          i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
-          if (DOC) {
-            eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
-            rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+            for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
           }
+          if (need_mask) {
+            asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int i = rowv[t];
-            const bool keep = (i >= 0) && (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
-            s[4 * q4 + t] = keep ? s[4 * q4 + t] : 0.f;
+            for (int q4 = 0; q4 < 4; ++q4) {
+              const int i0 = 32 * qb + 8 * q4 + 4 * g;
+              i32x4 eqv = {0, 0, 0, 0};
+              i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
+              if (DOC) {
+                eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+                rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+              }
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const int i = rowv[t];
+                const bool keep = (i >= 0) && (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
+                x[4 * q4 + t] = keep ? x[4 * q4 + t] : 0.f;
+              }
+            }
+          }
+          // hand P to the gradient wave of the pair (same lane, same register order)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 pv = {x[4 * q4], x[4 * q4 + 1], x[4 * q4 + 2], x[4 * q4 + 3]};
+            *reinterpret_cast<f32x4*>(pbuf + q4 * 1024) = pv;
           }
         }
       }
-      // dp -> dS = P * (dP - delta)
+      __syncthreads();
+      if (!skip) {
+        if (role == 1) {
+          // dS = P * (dP - delta)
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int i0 = 32 * qb + 8 * q4 + 4 * g;
-        const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const int i0 = 32 * qb + 8 * q4 + 4 * g;
+            const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+            const f32x4 pv = *reinterpret_cast<const f32x4*>(pbuf + q4 * 1024);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) dp[4 * q4 + t] = s[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
-      }
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        vec8 pf, dsf;
-#pragma unroll
-        for (int t = 0; t < 8; t += 2) {
-          const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
-          const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
-          pf[t] = pr[0]; pf[t + 1] = pr[1];
-          dsf[t] = dr[0]; dsf[t + 1] = dr[1];
+            for (int t = 0; t < 4; ++t) x[4 * q4 + t] = pv[t] * (x[4 * q4 + t] - dl[t]);
+          }
         }
-        const int goff = (2 * qb + half) * 16 * DL * 2;
+        // second product: dV^T += dO^T P (score wave) or dK^T += Q^T dS (gradient wave)
 #pragma unroll
-        for (int db = 0; db < DBN; ++db) {
-          const vec8 dot = lds_tr8<E>(ldo + lo.tr[db][0] + goff, ldo + lo.tr[db][1] + goff);
-          dv[db] = E::mfma32(dot, pf, dv[db]);
-        }
+        for (int half = 0; half < 2; ++half) {
+          vec8 yf;
 #pragma unroll
-        for (int db = 0; db < DBN; ++db) {
-          const vec8 qtf = lds_tr8<E>(lqt + lo.tr[db][0] + goff, lqt + lo.tr[db][1] + goff);
-          dk[db] = E::mfma32(qtf, dsf, dk[db]);
+          for (int t = 0; t < 8; t += 2) {
+            const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
+            yf[t] = pr[0]; yf[t + 1] = pr[1];
+          }
+          const int goff = (2 * qb + half) * 16 * DL * 2;
+#pragma unroll
+          for (int db = 0; db < DBN; ++db) {
+            const vec8 tf = lds_tr8<E>(t2 + lo.tr[db][0] + goff, t2 + lo.tr[db][1] + goff);
+            acc[db] = E::mfma32(tf, yf, acc[db]);
+          }
         }
       }
     }
@@ -280,37 +291,31 @@ void bwd_dkdv_kernel(const KArgs a) {
       compute(1, cur);
       cur = nxt; nxt = nxt2;
     }
-
   }
 
   if (key < a.N) {
-    T* krow = dkp + int64_t(key) * a.dk_rs;
-    T* vrow = dvp + int64_t(key) * a.dv_rs;
-    const float sc = a.scale;
+    T* orow = role == 0 ? reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs
+                        : reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
+    const float sc = role == 0 ? 1.0f : a.scale;
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
-        const typename E::vec2 k0 = E::cvt2(dk[db][4 * q4 + 0] * sc, dk[db][4 * q4 + 1] * sc);
-        const typename E::vec2 k1 = E::cvt2(dk[db][4 * q4 + 2] * sc, dk[db][4 * q4 + 3] * sc);
-        const typename E::vec2 v0 = E::cvt2(dv[db][4 * q4 + 0], dv[db][4 * q4 + 1]);
-        const typename E::vec2 v1 = E::cvt2(dv[db][4 * q4 + 2], dv[db][4 * q4 + 3]);
+        const typename E::vec2 k0 = E::cvt2(acc[db][4 * q4 + 0] * sc, acc[db][4 * q4 + 1] * sc);
+        const typename E::vec2 k1 = E::cvt2(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc);
         typename E::vec4 xk = {k0[0], k0[1], k1[0], k1[1]};
-        typename E::vec4 xv = {v0[0], v0[1], v1[0], v1[1]};
-        *reinterpret_cast<typename E::vec4*>(krow + 32 * db + 8 * q4 + 4 * g) = xk;
-        *reinterpret_cast<typename E::vec4*>(vrow + 32 * db + 8 * q4 + 4 * g) = xv;
+        *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = xk;
       }
   }
 }
-
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BK = 128, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
   const int slots = (a.B * a.Hk + 7) / 8;
-  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024;
+  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + 8 * 4096;
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -318,7 +323,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(8 * slots * nKt), dim3(256), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(8 * slots * nKt), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 

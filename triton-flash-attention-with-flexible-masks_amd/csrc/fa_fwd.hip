@@ -97,16 +97,35 @@ void fwd_kernel(const KArgs a) {
     if (skip) return;
 
     f32x16 s[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    __builtin_amdgcn_sched_barrier(0);
+    // The two 32-key blocks are accumulated alternately: an MFMA that accumulates onto the result
+    // of the MFMA issued right before it waits a full extra MFMA time, two interleaved chains do not.
+    {
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      s[kb] = zero;
+      s[0] = zero;
+      s[1] = zero;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
-        s[kb] = E::mfma32(kf, qf[ks], s[kb]);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
+          s[kb] = E::mfma32(kf, qf[ks], s[kb]);
+        }
       }
     }
+    // Instruction order of this region: keep several K fragments in flight ahead of the MFMA that
+    // consumes them (an LDS read takes about as long as three MFMAs).
+    {
+      constexpr int NQK = 2 * KS, PRE = NQK < 4 ? NQK : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+      for (int i = 0; i < NQK - PRE; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (need_mask) {
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
 #pragma unroll
@@ -158,6 +177,7 @@ void fwd_kernel(const KArgs a) {
     }
     l_run += ps0 + ps1;
     // O^T += V^T P^T, 16 keys per MFMA
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int c16 = 0; c16 < 4; ++c16) {
       vec8 pf;
@@ -173,6 +193,18 @@ void fwd_kernel(const KArgs a) {
         o[db] = E::mfma32(vf, pf, o[db]);
       }
     }
+    // V^T fragments (two transposed reads each) four MFMAs ahead; P conversions just in time
+    {
+      constexpr int NPV = 4 * DBN, PRE = NPV < 4 ? NPV : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
+#pragma unroll
+      for (int i = 0; i < NPV; ++i) {
+        if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i < NPV - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   int cur = it.next();

@@ -137,3 +137,90 @@ def flops(w: Workload, mode: str = "fwd", kept=None, tiles=None, tile: int = 128
         "elem": 4.0 * w.D * w.H * kept * mult,
         "tile": 4.0 * w.D * w.H * tile * tile * tiles * mult,
     }
+
+
+# ---------------------------------------------------------------------------
+# Executed work: a host emulation of the tile decisions the kernels take (mask plan,
+# permuted order, per-wave skip tests), so that reports can state the FLOPs the MFMA
+# pipes really execute next to the algorithmic (mask-derived) counts.
+# ---------------------------------------------------------------------------
+_IMAX, _IMIN = 2**31 - 1, -2**31
+
+
+def _summaries(ids, rows, n):
+    """Per group of n entries of `rows` (row indices, -1 = none): lo/hi over local ids, glob, rmin, rmax."""
+    G = len(rows) // n
+    r = rows.reshape(G, n)
+    valid = r >= 0
+    v = np.where(valid, ids[np.maximum(r, 0)], 0)
+    local = valid & (v < 0)
+    lo = np.where(local, v, _IMAX).min(1)
+    hi = np.where(local, v, _IMIN).max(1)
+    glob = (valid & (v >= 0)).any(1)
+    rmin = np.where(valid, r, _IMAX).min(1)
+    rmax = np.where(valid, r, -1).max(1)
+    return lo, hi, glob, rmin, rmax, valid.sum(1)
+
+
+def executed_wave_steps(w: Workload):
+    """(forward/dq wave steps, dk/dv wave steps) per head, summed over the batch.
+
+    A forward (or dq) wave step is 32 query rows x 64 keys; a dk/dv wave step is 64 query rows x
+    32 keys.  Both cover 2048 score elements, i.e. 2048 * 4 * D FLOPs in the forward.
+    """
+    gap = max(0, w.Lk - w.Lq)
+    fwd_steps = kv_steps = 0
+    nK64 = (w.Lk + 63) // 64
+    nK32 = (w.Lk + 31) // 32
+    for b in range(w.B):
+        if w.doc:
+            eq = w.eq[b].astype(np.int64)
+            ek = w.ek[b].astype(np.int64)
+            local = np.nonzero(eq < 0)[0]
+            glob = np.nonzero(eq >= 0)[0]
+            nLp = (len(local) + 255) // 256 * 256
+            Pp = (w.Lq + 255) // 256 * 256 + 256
+            perm = np.full(Pp, -1, np.int64)
+            perm[:len(local)] = local
+            perm[nLp:nLp + len(glob)] = glob
+        else:
+            eq = np.zeros(w.Lq, np.int64)         # every row "global": no doc test
+            ek = np.zeros(w.Lk, np.int64)
+            Pp = (w.Lq + 127) // 128 * 128
+            perm = np.where(np.arange(Pp) < w.Lq, np.arange(Pp), -1)
+        pad = lambda x, n, fill: np.concatenate([x, np.full(n - len(x), fill, x.dtype)])
+        k64 = pad(ek, nK64 * 64, 0).reshape(nK64, 64)
+        kvalid64 = (np.arange(nK64 * 64).reshape(nK64, 64) < w.Lk)
+        k64_lo = np.where(kvalid64, k64, _IMAX).min(1)
+        k64_hi = np.where(kvalid64, k64, _IMIN).max(1)
+        # forward / dq: waves of 32 rows against key tiles of 64
+        lo, hi, g, rmin, rmax, nv = _summaries(eq, perm, 32)
+        j0 = np.arange(nK64)[None, :] * 64
+        vis = np.broadcast_to(nv[:, None] > 0, (len(nv), nK64)).copy()
+        if w.causal:
+            vis = vis & (j0 <= gap + rmax[:, None])
+        if w.doc:
+            vis = vis & (g[:, None] | ((lo[:, None] <= k64_hi[None, :]) & (k64_lo[None, :] <= hi[:, None])))
+        fwd_steps += int(vis.sum())
+        # dk/dv: waves of 32 keys against query tiles of 64 (permuted order)
+        k32 = pad(ek, nK32 * 32, 0).reshape(nK32, 32)
+        kvalid32 = (np.arange(nK32 * 32).reshape(nK32, 32) < w.Lk)
+        k32_lo = np.where(kvalid32, k32, _IMAX).min(1)
+        k32_hi = np.where(kvalid32, k32, _IMIN).max(1)
+        perm64 = pad(perm, (len(perm) + 63) // 64 * 64, -1)
+        lo, hi, g, rmin, rmax, nv = _summaries(eq, perm64, 64)
+        n0 = np.arange(nK32)[None, :] * 32
+        vis = np.broadcast_to(nv[:, None] > 0, (len(nv), nK32)).copy()
+        if w.causal:
+            vis = vis & (gap + rmax[:, None] >= n0)
+        if w.doc:
+            vis = vis & (g[:, None] | ((lo[:, None] <= k32_hi[None, :]) & (k32_lo[None, :] <= hi[:, None])))
+        kv_steps += int(vis.sum())
+    return fwd_steps, kv_steps
+
+
+def executed_flops(w: Workload):
+    """FLOPs the MFMA pipes execute per kernel: forward (2 GEMMs), dq (3), dk/dv (4)."""
+    f, kv = executed_wave_steps(w)
+    unit = 2048 * 4.0 * w.D * w.H     # one wave step, forward accounting
+    return {"fwd": f * unit, "dq": 1.5 * f * unit, "dkdv": 2.0 * kv * unit}
