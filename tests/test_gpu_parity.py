@@ -128,6 +128,16 @@ def test_all_global_and_all_local_ids():
     _run_case(1, 2, 2, 256, 256, 128, torch.bfloat16, True, True, seed=6, ids_kind="alllocal")
 
 
+def test_long_key_ranges_of_global_rows():
+    # Rows with id >= 0 see long key ranges; tiles of such rows are cut into key chunks that
+    # separate workgroups process and merge.  Covers 2 and 4 chunks, causal and not, a ragged
+    # last key tile, and more global-row tiles than the number that is ever cut.
+    _run_case(1, 2, 2, 4096, 4096, 64, torch.bfloat16, True, True, seed=21)
+    _run_case(1, 2, 1, 300, 5000, 128, torch.float16, False, True, seed=22)
+    _run_case(1, 1, 1, 1200, 2304, 128, torch.bfloat16, True, True, seed=23, ids_kind="allglobal")
+    _run_case(2, 2, 2, 2048, 2048, 16, torch.bfloat16, True, True, seed=24)
+
+
 def test_per_head_int64_ids():
     _run_case(1, 3, 3, 192, 192, 64, torch.bfloat16, True, True, seed=9, per_head_ids=True, id_dtype=torch.int64)
 
@@ -188,7 +198,11 @@ def test_device_mask_plan_matches_host_restatement():
     o_hd = off; off += r256(B * H * 16)
     o_qs = off; off += r256(B * H * nQs * 32)
     o_ks = off; off += r256(B * H * nKs * 32)
+    # scratch of the split global-row tiles: arrival counters, (max, sum) pairs, fp32 partials
+    o_sc = off; off += r256(B * H * 8 * 4)
+    off += r256(B * H * 8 * 4 * 128 * 2 * 4) + r256(B * H * 8 * 4 * 128 * D * 4)
     assert off == ws.size
+    assert not ws[o_sc:o_sc + B * H * 8 * 4].any()   # the plan leaves the counters at zero
     i32 = lambda o, n: ws[o:o + 4 * n].view(np.int32)
     perm = i32(o_pm, B * H * Pp).reshape(B, H, Pp)
     peq = i32(o_pq, B * H * Pp).reshape(B, H, Pp)

@@ -148,8 +148,12 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
 // bound), so that the compute kernels start their tile search in the right place.
 __global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal_gap,
                                                         const int* __restrict__ perm, const int* __restrict__ peq,
-                                                        const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum) {
+                                                        const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum,
+                                                        int* __restrict__ sk_cnt, int n_sk) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the arrival counters of the split-key merge start every forward at zero
+  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)
+    for (int i = threadIdx.x; i < n_sk; i += 256) sk_cnt[i] = 0;
   const int t = blockIdx.x * 4 + wave;
   if (t >= nQs) return;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -222,7 +226,8 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     const int gap = p->N > p->M ? p->N - p->M : 0;
     hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
-                       p->causal ? gap : -1, perm, peq, ksum, qsum);
+                       p->causal ? gap : -1, perm, peq, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
+                       p->B * p->H * kSplitTiles);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   return 0;

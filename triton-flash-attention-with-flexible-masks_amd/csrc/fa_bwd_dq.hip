@@ -29,11 +29,17 @@ void bwd_dq_kernel(const KArgs a) {
   const int g = lane >> 5;
 
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
+  const int nSlots = nQt + (DOC ? kSplitExtra : 0);
   int slot, bh;
-  if (!block_to_tile(nQt, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
+  if (!block_to_tile(nSlots, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  QWork wk;
+  if (!q_work<DOC>(a, b, h, nQt, slot, wk)) return;
   QTileCtx<CAUSAL, DOC> qc;
-  if (!qc.init(a, b, h, nQt - 1 - slot, threadIdx.x >> 6)) return;
+  if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
+  int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
+  const int nsplit = split_range(wk, kt_first, kt_last);
+  if (wk.split >= nsplit) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
 
@@ -57,7 +63,7 @@ void bwd_dq_kernel(const KArgs a) {
   const float delta_i = delp[rowc];
 
   TileIter it;
-  it.init_keys(qc.first_tile(), qc.last_tile(a), qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
@@ -158,6 +164,43 @@ void bwd_dq_kernel(const KArgs a) {
     cur = nxt;
   }
 
+  if (DOC && nsplit > 1) {
+    // This workgroup saw one chunk of the keys: store the partial sum; the last chunk to arrive
+    // adds them up in a fixed order and writes dQ.
+    const int64_t tbase = (int64_t(b) * a.H + h) * kSplitTiles + wk.gt;
+    float* po = a.sk_o + (tbase * kSplitK + wk.split) * (128 * D);
+    const int rt = (threadIdx.x >> 6) * 32 + (lane & 31);   // row inside the tile
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        if (32 * db + 8 * q4 >= D) continue;
+        f32x4 x = {dq[db][4 * q4 + 0], dq[db][4 * q4 + 1], dq[db][4 * q4 + 2], dq[db][4 * q4 + 3]};
+        store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
+      }
+    if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
+    constexpr int C4 = D / 4;
+    const float* bo = a.sk_o + tbase * kSplitK * (128 * D);
+    const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
+    for (int i = threadIdx.x; i < 128 * C4; i += 256) {
+      const int r = i / C4, c = i % C4;
+      const int mrow = prm[r];
+      if (mrow < 0) continue;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sp = 0; sp < kSplitK; ++sp) {
+        if (sp >= nsplit) continue;
+        const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
+        acc[0] += x[0]; acc[1] += x[1]; acc[2] += x[2]; acc[3] += x[3];
+      }
+      const typename E::vec2 x0 = E::cvt2(acc[0] * a.scale, acc[1] * a.scale);
+      const typename E::vec2 x1 = E::cvt2(acc[2] * a.scale, acc[3] * a.scale);
+      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
+      *reinterpret_cast<typename E::vec4*>(dqp + int64_t(mrow) * a.dq_rs + 4 * c) = x;
+    }
+    return;
+  }
+
   if (row >= 0) {
     T* drow = dqp + int64_t(row) * a.dq_rs;
     const float sc = a.scale;
@@ -178,7 +221,7 @@ void bwd_dq_kernel(const KArgs a) {
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
-  const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
+  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? kSplitExtra : 0);
   const int slots = (a.B * a.H + 7) / 8;
   const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2;
   auto kern = bwd_dq_kernel<Tag, D, CAUSAL, DOC>;

@@ -41,6 +41,14 @@ constexpr int kSumRows = 64;
 // The local-row part of the permuted order is padded to this many entries, so that a
 // workgroup of up to 256 query rows never mixes local and global rows.
 constexpr int kPermAlign = 256;
+// Tiles of global rows (eq >= 0) see every key up to their own position, i.e. up to the whole
+// sequence: a single workgroup walking 16K keys is the critical path of the kernel.  The key range
+// of the first kSplitTiles such tiles of a (batch, head) is therefore cut into up to kSplitK chunks
+// handled by different workgroups; each writes an fp32 partial result and the last one to arrive
+// (an atomic counter per tile) merges them.  The merge order is fixed, results stay reproducible.
+constexpr int kSplitK = 4;
+constexpr int kSplitTiles = 8;
+constexpr int kSplitMinTiles = 16;   // key tiles (of 64) per chunk below which splitting does not pay
 
 struct bf16_t {};
 struct fp16_t {};
@@ -178,6 +186,10 @@ struct KArgs {
   const QHeader* qhdr;    // [B, Hq']
   const IdSummary* qsum;  // [B, Hq', nQs]  per 64 entries of the permuted order
   const IdSummary* ksum;  // [B, Hk', nKs]  per 64 keys
+  // split-key scratch of the global-row tiles, see kSplitK: per (b, h, global tile g)
+  int* sk_cnt;            // [B, H, kSplitTiles]              arrival counters (zero between kernels)
+  float* sk_ml;           // [B, H, kSplitTiles, kSplitK, 128, 2]  per row: reference point, row sum
+  float* sk_o;            // [B, H, kSplitTiles, kSplitK, 128, D]  per row: unnormalised partial result
   int64_t q_bs, q_hs, q_rs;
   int64_t k_bs, k_hs, k_rs;
   int64_t v_bs, v_hs, v_rs;
@@ -206,7 +218,8 @@ struct WsLayout {
   int Pp;                 // length of the permuted order
   int nQs, nKs;
   int nCh;                // row chunks of the partition kernels
-  uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum, total;  // bytes
+  uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum;  // bytes
+  uint64_t off_sk_cnt, off_sk_ml, off_sk_o, total;
 };
 
 inline WsLayout ws_layout(const fa_params* p) {
@@ -229,6 +242,10 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_qhdr = take(uint64_t(p->B) * w.Hq1 * sizeof(QHeader));
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
+  const uint64_t nsk = uint64_t(p->B) * p->H * kSplitTiles;
+  w.off_sk_cnt = take(nsk * 4);
+  w.off_sk_ml = take(nsk * kSplitK * 128 * 2 * 4);
+  w.off_sk_o = take(nsk * kSplitK * 128 * uint64_t(p->D) * 4);
   w.total = o;
   return w;
 }

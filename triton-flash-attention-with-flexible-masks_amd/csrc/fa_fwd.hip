@@ -43,11 +43,17 @@ void fwd_kernel(const KArgs a) {
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
   // order and see the longest key ranges; without ids the last rows do
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
+  const int nSlots = nQt + (DOC ? kSplitExtra : 0);
   int slot, bh;
-  if (!block_to_tile(nQt, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
+  if (!block_to_tile(nSlots, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  QWork wk;
+  if (!q_work<DOC>(a, b, h, nQt, slot, wk)) return;
   QTileCtx<CAUSAL, DOC> qc;
-  if (!qc.init(a, b, h, nQt - 1 - slot, threadIdx.x >> 6)) return;
+  if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
+  int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
+  const int nsplit = split_range(wk, kt_first, kt_last);
+  if (wk.split >= nsplit) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
 
@@ -70,7 +76,7 @@ void fwd_kernel(const KArgs a) {
   }
 
   TileIter it;
-  it.init_keys(qc.first_tile(), qc.last_tile(a), qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
@@ -234,8 +240,62 @@ void fwd_kernel(const KArgs a) {
     cur = nxt;
   }
 
-  // epilogue: normalise, write O and LSE
   const float l_tot = xhalf_sum(l_run);
+  if (DOC && nsplit > 1) {
+    // This workgroup saw one chunk of the keys: store the unnormalised partial result; the last
+    // chunk to arrive combines them (log-sum-exp merge) and writes O and LSE.
+    const int64_t tbase = (int64_t(b) * a.H + h) * kSplitTiles + wk.gt;
+    float* po = a.sk_o + (tbase * kSplitK + wk.split) * (128 * D);
+    float* pml = a.sk_ml + (tbase * kSplitK + wk.split) * (128 * 2);
+    const int rt = (threadIdx.x >> 6) * 32 + (lane & 31);   // row inside the tile
+    if (g == 0) store_dev(pml + rt * 2, m_ref, l_tot);
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        if (32 * db + 8 * q4 >= D) continue;
+        f32x4 x = {o[db][4 * q4 + 0], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]};
+        store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
+      }
+    if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
+    // merge: the whole workgroup walks the tile, one float4 of one row per thread and step
+    constexpr int C4 = D / 4;
+    const float* bo = a.sk_o + tbase * kSplitK * (128 * D);
+    const float* bml = a.sk_ml + tbase * kSplitK * (128 * 2);
+    const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
+    for (int i = threadIdx.x; i < 128 * C4; i += 256) {
+      const int r = i / C4, c = i % C4;
+      const int mrow = prm[r];
+      if (mrow < 0) continue;
+      float ms[kSplitK], ls[kSplitK], mmax = -INFINITY;
+#pragma unroll
+      for (int sp = 0; sp < kSplitK; ++sp) {
+        const bool on = sp < nsplit;
+        ms[sp] = -INFINITY; ls[sp] = 0.f;
+        if (on) load_dev(bml + sp * 256 + r * 2, ms[sp], ls[sp]);
+        mmax = fmaxf(mmax, ms[sp]);
+      }
+      float lsum = 0.f;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sp = 0; sp < kSplitK; ++sp) {
+        if (sp >= nsplit) continue;
+        const float w = ms[sp] == -INFINITY ? 0.f : fast_exp2(ms[sp] - mmax);
+        lsum += w * ls[sp];
+        const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
+        acc[0] += w * x[0]; acc[1] += w * x[1]; acc[2] += w * x[2]; acc[3] += w * x[3];
+      }
+      const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+      if (c == 0) lsep[mrow] = lsum > 0.f ? mmax + fast_log2(lsum) : -INFINITY;
+      const typename E::vec2 x0 = E::cvt2(acc[0] * inv, acc[1] * inv);
+      const typename E::vec2 x1 = E::cvt2(acc[2] * inv, acc[3] * inv);
+      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
+      *reinterpret_cast<typename E::vec4*>(op + int64_t(mrow) * a.o_rs + 4 * c) = x;
+    }
+    return;
+  }
+
+  // epilogue: normalise, write O and LSE
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   if (row >= 0) {
     if (g == 0) lsep[row] = l_tot > 0.f ? m_ref + fast_log2(l_tot) : -INFINITY;
@@ -253,11 +313,10 @@ void fwd_kernel(const KArgs a) {
   }
 }
 
-
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
-  const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
+  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? kSplitExtra : 0);
   const int slots = (a.B * a.H + 7) / 8;
   const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2;
   auto kern = fwd_kernel<Tag, D, CAUSAL, DOC>;

@@ -284,6 +284,92 @@ struct QTileCtx {
   }
 };
 
+// ---------------------------------------------------------------------------
+// Work assignment of one workgroup of the forward / dq kernels, including the split of the
+// key range of global-row tiles (kSplitK, fa_common.h).
+//   slots [0, nE)          : chunks 1 .. kSplitK-1 of the first kSplitTiles global-row tiles
+//   slots [nE, nE + nQt)   : every tile, last tile first (chunk 0 when the tile is split)
+// ---------------------------------------------------------------------------
+struct QWork {
+  int tile;    // 128-row tile (natural order, or permuted order with ids)
+  int gt;      // index among the splittable global-row tiles, or -1
+  int split;   // chunk of the key range handled by this workgroup
+};
+constexpr int kSplitExtra = kSplitTiles * (kSplitK - 1);
+
+template <bool DOC>
+FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
+  if (!DOC) { w.tile = nQt - 1 - slot; w.gt = -1; w.split = 0; return true; }
+  const QHeader hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
+  const int g0 = hd.nLp / 128;   // first global-row tile
+  if (slot < kSplitExtra) {
+    w.gt = slot / (kSplitK - 1);
+    w.split = 1 + slot % (kSplitK - 1);
+    w.tile = g0 + w.gt;
+    return w.tile < hd.nT128;
+  }
+  w.tile = nQt - 1 - (slot - kSplitExtra);
+  w.split = 0;
+  w.gt = (w.tile >= g0 && w.tile - g0 < kSplitTiles) ? w.tile - g0 : -1;
+  return true;
+}
+
+// Cut the key-tile range [first, last) of a splittable tile into chunks; returns the number of
+// chunks in use (1: not split) and narrows [first, last) to this workgroup's chunk.
+FA_DEV int split_range(const QWork& w, int& first, int& last) {
+  if (w.gt < 0) return 1;
+  const int n = max(0, last - first);
+  const int ns = min(kSplitK, max(1, n / kSplitMinTiles));
+  const int c = (n + ns - 1) / ns;
+  first = min(last, first + w.split * c);
+  last = min(last, first + c);
+  return ns;
+}
+
+// Partial results travel between workgroups through device-scope accesses (they pass the
+// non-coherent cache levels access by access), so no cache-wide write-back or invalidate is needed.
+FA_DEV void store_dev(float* p, float x0, float x1) {
+  typedef unsigned long long u64;
+  const u64 v = (u64)__float_as_uint(x0) | ((u64)__float_as_uint(x1) << 32);
+  __hip_atomic_store(reinterpret_cast<u64*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+FA_DEV void store_dev(float* p, f32x4 x) {
+  // elements go through scalars: a bit cast applied to a vector element reads element 0
+  const float x0 = x[0], x1 = x[1], x2 = x[2], x3 = x[3];
+  store_dev(p, x0, x1);
+  store_dev(p + 2, x2, x3);
+}
+FA_DEV void load_dev(const float* p, float& x0, float& x1) {
+  typedef unsigned long long u64;
+  const u64 v = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  x0 = __uint_as_float((unsigned)v);
+  x1 = __uint_as_float((unsigned)(v >> 32));
+}
+FA_DEV f32x4 load_dev4(const float* p) {
+  float a, b, c, d;
+  load_dev(p, a, b);
+  load_dev(p + 2, c, d);
+  const f32x4 x = {a, b, c, d};
+  return x;
+}
+
+// Arrival protocol of the chunks of one tile: every workgroup calls this after it has issued the
+// stores of its partial result (store_dev); returns true in exactly one of them, the last to
+// arrive, which then merges (load_dev).
+FA_DEV bool split_arrive(int* counter, int nsplit) {
+  __shared__ int sk_last;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial stores have landed
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sk_last = (old == nsplit - 1) ? 1 : 0;
+    // ready for the next kernel that uses the same scratch
+    if (sk_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  return sk_last != 0;
+}
+
 // blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head).
 // Consecutive workgroup ids land on different XCDs, so every XCD is given whole
 // heads (its L2 then keeps that head's K/V or Q/dO).  Inside an XCD the order is
