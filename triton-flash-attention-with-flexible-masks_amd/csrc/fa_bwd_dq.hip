@@ -77,12 +77,13 @@ void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-  auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int k_lo, const int k_hi) __attribute__((always_inline)) {
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
+    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
     const int n0 = cur * BN;
-    bool skip, need_mask;
-    qc.decide(a, cur, n0, BN, skip, need_mask);
+    bool skip, need_lim, need_doc;
+    qc.decide(a, n0, BN, k_lo, k_hi, skip, need_lim, need_doc);
     if (skip) return;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -104,19 +105,13 @@ void bwd_dq_kernel(const KArgs a) {
         const float p = fast_exp2(__builtin_fmaf(s[r], c, -L_i));
         s[r] = p * (dp[r] - delta_i);
       }
-      if (need_mask) {
+      if (need_lim) {
         asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int j0 = n0 + 32 * kb + 8 * q4 + 4 * g;
-          i32x4 ekv = {0, 0, 0, 0};
-          if (DOC) ekv = *reinterpret_cast<const i32x4*>(ekp + j0);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const bool keep = keep_elem<CAUSAL, DOC>(row, j0 + t, a.gap, a.N, eq_i, ekv[t]);
-            s[4 * q4 + t] = keep ? s[4 * q4 + t] : 0.f;
-          }
-        }
+        mask_lim(s, qc.lim_i - n0 - 32 * kb - 4 * g, 0.f);
+      }
+      if (DOC && need_doc) {
+        asm volatile("" ::: "memory");
+        mask_doc(s, lid + kb * 32 * 4, eq_i, qc.glob_i, 0.f);
       }
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
@@ -137,31 +132,30 @@ void bwd_dq_kernel(const KArgs a) {
     }
   };
 
+  // tile streams: K, V and (with ids) the 64 key ids of the tile, all straight into LDS
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  auto issue = [&](const int BUF, const int t) __attribute__((always_inline)) {
+    ldK.issue(t * BN, smem + BUF * TILE_BYTES);
+    ldV.issue(t * BN, smem + (2 + BUF) * TILE_BYTES);
+    if (DOC && wave == 0) glb_load_lds4(ekp + t * BN + lane, smem + 4 * TILE_BYTES + BUF * (BN * 4));
+  };
   int cur = it.next();
-  if (cur >= 0) {
-    ldK.issue(cur * BN, smem + 0 * TILE_BYTES);
-    ldV.issue(cur * BN, smem + 2 * TILE_BYTES);
-  }
+  int cur_lo = it.t_lo, cur_hi = it.t_hi;
+  if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
     int nxt = it.next();
     wait_async_loads();
     __syncthreads();
-    if (nxt >= 0) {
-      ldK.issue(nxt * BN, smem + 1 * TILE_BYTES);
-      ldV.issue(nxt * BN, smem + 3 * TILE_BYTES);
-    }
-    compute(0, cur);
-    cur = nxt;
+    if (nxt >= 0) issue(1, nxt);
+    compute(0, cur, cur_lo, cur_hi);
+    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
     if (cur < 0) break;
     nxt = it.next();
     wait_async_loads();
     __syncthreads();
-    if (nxt >= 0) {
-      ldK.issue(nxt * BN, smem + 0 * TILE_BYTES);
-      ldV.issue(nxt * BN, smem + 2 * TILE_BYTES);
-    }
-    compute(1, cur);
-    cur = nxt;
+    if (nxt >= 0) issue(0, nxt);
+    compute(1, cur, cur_lo, cur_hi);
+    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
   }
 
   if (DOC && nsplit > 1) {
@@ -223,7 +217,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
   const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? kSplitExtra : 0);
   const int slots = (a.B * a.H + 7) / 8;
-  const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2;
+  const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2 + 2 * BN * 4;  // K, V double buffered + key ids
   auto kern = bwd_dq_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {

@@ -37,7 +37,7 @@ void fwd_kernel(const KArgs a) {
   constexpr float RESCALE_THRESH = 8.0f;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 5;
 
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
@@ -93,13 +93,14 @@ void fwd_kernel(const KArgs a) {
   float l_run = 0.f;        // this lane's partial row sum
 
   // One K/V tile; BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int k_lo, const int k_hi) __attribute__((always_inline)) {
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
+    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
     const int n0 = cur * BN;
 
-    bool skip, need_mask;
-    qc.decide(a, cur, n0, BN, skip, need_mask);
+    bool skip, need_lim, need_doc;
+    qc.decide(a, n0, BN, k_lo, k_hi, skip, need_lim, need_doc);
     if (skip) return;
 
     f32x16 s[2];
@@ -132,22 +133,16 @@ void fwd_kernel(const KArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (need_mask) {
+    if (need_lim) {
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int j0 = n0 + 32 * kb + 8 * q4 + 4 * g;
-          i32x4 ekv = {0, 0, 0, 0};
-          if (DOC) ekv = *reinterpret_cast<const i32x4*>(ekp + j0);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const bool keep = keep_elem<CAUSAL, DOC>(row, j0 + t, a.gap, a.N, eq_i, ekv[t]);
-            s[kb][4 * q4 + t] = keep ? s[kb][4 * q4 + t] : -INFINITY;
-          }
-        }
-      }
+      const int rel = qc.lim_i - n0 - 4 * g;
+      mask_lim(s[0], rel, -INFINITY);
+      mask_lim(s[1], rel - 32, -INFINITY);
+    }
+    if (DOC && need_doc) {
+      asm volatile("" ::: "memory");
+      mask_doc(s[0], lid, eq_i, qc.glob_i, -INFINITY);
+      mask_doc(s[1], lid + 32 * 4, eq_i, qc.glob_i, -INFINITY);
     }
     // online softmax in the exp2 domain with a lazily moved reference point
     float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
@@ -213,31 +208,29 @@ void fwd_kernel(const KArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  // tile streams: K, V and (with ids) the 64 key ids of the tile, all straight into LDS
+  auto issue = [&](const int BUF, const int t) __attribute__((always_inline)) {
+    ldK.issue(t * BN, smem + BUF * TILE_BYTES);
+    ldV.issue(t * BN, smem + (2 + BUF) * TILE_BYTES);
+    if (DOC && wave == 0) glb_load_lds4(ekp + t * BN + lane, smem + 4 * TILE_BYTES + BUF * (BN * 4));
+  };
   int cur = it.next();
-  if (cur >= 0) {
-    ldK.issue(cur * BN, smem + 0 * TILE_BYTES);
-    ldV.issue(cur * BN, smem + 2 * TILE_BYTES);
-  }
+  int cur_lo = it.t_lo, cur_hi = it.t_hi;
+  if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
     int nxt = it.next();
     wait_async_loads();
     __syncthreads();
-    if (nxt >= 0) {
-      ldK.issue(nxt * BN, smem + 1 * TILE_BYTES);
-      ldV.issue(nxt * BN, smem + 3 * TILE_BYTES);
-    }
-    compute(0, cur);
-    cur = nxt;
+    if (nxt >= 0) issue(1, nxt);
+    compute(0, cur, cur_lo, cur_hi);
+    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
     if (cur < 0) break;
     nxt = it.next();
     wait_async_loads();
     __syncthreads();
-    if (nxt >= 0) {
-      ldK.issue(nxt * BN, smem + 0 * TILE_BYTES);
-      ldV.issue(nxt * BN, smem + 2 * TILE_BYTES);
-    }
-    compute(1, cur);
-    cur = nxt;
+    if (nxt >= 0) issue(0, nxt);
+    compute(1, cur, cur_lo, cur_hi);
+    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
   }
 
   const float l_tot = xhalf_sum(l_run);
@@ -318,7 +311,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
   const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? kSplitExtra : 0);
   const int slots = (a.B * a.H + 7) / 8;
-  const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2;
+  const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2 + 2 * BN * 4;  // K, V double buffered + key ids
   auto kern = fwd_kernel<Tag, D, CAUSAL, DOC>;
   static bool attr_set = false;
   if (!attr_set) {

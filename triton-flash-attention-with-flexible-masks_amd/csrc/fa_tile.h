@@ -84,7 +84,7 @@ struct TileLoader {
   static constexpr int NI = ROWS / RPI;  // wave instructions per tile
   static constexpr int PER = (NI + NW - 1) / NW;  // per wave (NW waves share the tile)
   buf_rsrc_t rsrc;
-  int voff[PER];
+  int voff;       // this lane's byte offset inside the first group of NW * RPI rows
   int row_bytes;
 
   // base: first row of the (batch, head) slice; rs: row stride in elements
@@ -93,20 +93,21 @@ struct TileLoader {
     const unsigned bytes = (unsigned)((int64_t(nrows - 1) * rs + GD) * 2);
     rsrc = make_rsrc(base, bytes);
     row_bytes = int(rs) * 2;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int row = (i * NW + wave) * RPI + lane / CPR;
-      const int c = (lane % CPR) ^ swz<D, SWZ_ROW>(row);
-      voff[i] = c < GD / 8 ? row * row_bytes + c * 16 : kOobOffset;
-    }
+    // The swizzle of a row depends on the row modulo NW * RPI only (see swz), so the lanes of wave
+    // instruction i address the rows of instruction 0 moved down by i * NW * RPI rows: one vector
+    // offset serves every instruction, the rest is a scalar offset.
+    static_assert((NW * RPI) % 16 == 0, "swizzle period");
+    const int row = wave * RPI + lane / CPR;
+    const int c = (lane % CPR) ^ swz<D, SWZ_ROW>(row);
+    voff = c < GD / 8 ? row * row_bytes + c * 16 : kOobOffset;
   }
   // stream rows row0 .. row0+ROWS-1 into the tile at `lds`
   FA_DEV void issue(int row0, char* lds) const {
-    const int wave = threadIdx.x >> 6;
-    const int soff = row0 * row_bytes;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: LDS targets stay in SGPRs
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-      if (NI % NW == 0 || i * NW + wave < NI) buf_load_lds16(rsrc, lds + (i * NW + wave) * 1024, voff[i], soff);
+      if (NI % NW == 0 || i * NW + wave < NI)
+        buf_load_lds16(rsrc, lds + (i * NW + wave) * 1024, voff, (row0 + i * NW * RPI) * row_bytes);
   }
 };
 
@@ -161,6 +162,8 @@ FA_DEV typename E::vec8 lds_tr8(const char* p0, const char* p1) {
 struct TileIter {
   unsigned long long mask;
   int base, last;
+  int c_lo, c_hi;          // this lane's candidate (tile base + lane): its id range
+  int t_lo, t_hi;          // id range of the tile returned by the last next() (keys mode, with ids)
   int o_lo, o_hi, o_glob;
   int min_rmax;            // query mode: candidates need rmax >= min_rmax
   bool keys_mode;
@@ -175,15 +178,16 @@ struct TileIter {
     start(first, last_);
   }
   FA_DEV void start(int first, int last_) {
-    last = last_;
+    last = last_; c_lo = 0; c_hi = -1; t_lo = 0; t_hi = -1;
     base = (first / 64) * 64;
     mask = chunk_mask(base) & (~0ull << (first - base));
   }
-  FA_DEV unsigned long long chunk_mask(int b) const {
+  FA_DEV unsigned long long chunk_mask(int b) {
     const int t = b + (threadIdx.x & 63);
     bool v = t < last;
     if (sum != nullptr && v) {
       const IdSummary s = sum[t];
+      c_lo = s.lo; c_hi = s.hi;
       v = keys_mode ? doc_may_keep(o_lo, o_hi, o_glob, s.lo, s.hi)
                     : (s.nvalid > 0 && s.rmax >= min_rmax && doc_may_keep(s.lo, s.hi, s.glob, o_lo, o_hi));
     }
@@ -196,9 +200,13 @@ struct TileIter {
       if (base >= last) return -1;
       mask = chunk_mask(base);
     }
-    const int j = base + __builtin_ctzll(mask);
+    const int jl = __builtin_ctzll(mask);
     mask &= mask - 1;
-    return j;
+    if (sum != nullptr) {   // no memory access in the tile loop: the range comes out of the registers
+      t_lo = __builtin_amdgcn_readlane(c_lo, jl);
+      t_hi = __builtin_amdgcn_readlane(c_hi, jl);
+    }
+    return base + jl;
   }
 };
 
@@ -215,6 +223,9 @@ struct QTileCtx {
   int w_lo, w_hi, w_glob, w_rmin, w_rmax;  // this wave's 32 rows
   int g_lo, g_hi, g_glob, g_rmax;          // the workgroup's 128 rows
   int g_kfirst, g_klast;                   // key tiles (of 64) those rows can need, from the mask plan
+  int lim_i;                               // last key this lane's row may see (causal and length limit)
+  int w_limmin;                            // smallest such limit among the wave's rows
+  bool glob_i;                             // this lane's row has an id >= 0 (sees every id)
   const int* ekp;
   const IdSummary* ksum;
 
@@ -263,6 +274,9 @@ struct QTileCtx {
       w_glob = __builtin_amdgcn_ballot_w64(eq_i >= 0 && row >= 0) != 0;
     }
     rowc = row >= 0 ? row : 0;
+    lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;
+    w_limmin = CAUSAL ? min(a.gap + w_rmin, a.N - 1) : a.N - 1;
+    glob_i = eq_i >= 0;
     return true;
   }
   // range [first, last) of 64-key tiles the workgroup has to look at
@@ -272,17 +286,39 @@ struct QTileCtx {
     return min((hi_key + 63) / 64, g_klast + 1);
   }
 
-  // wave-level decisions for key tile `cur` (keys n0 .. n0+BN-1)
-  FA_DEV void decide(const KArgs& a, int cur, int n0, int BN, bool& skip, bool& need_mask) const {
+  // Wave-level decisions for the key tile n0 .. n0+BN-1 whose ids span [k_lo, k_hi]:
+  //   skip     : no (row, key) pair of the wave's rows is kept
+  //   need_lim : some pair fails the causal / length limit  -> mask_lim
+  //   need_doc : some pair may fail the id test             -> mask_doc
+  FA_DEV void decide(const KArgs& a, int n0, int BN, int k_lo, int k_hi, bool& skip, bool& need_lim, bool& need_doc) const {
     skip = (w_rmax < 0) || (CAUSAL && (n0 > a.gap + w_rmax));
-    need_mask = (n0 + BN > a.N) || (CAUSAL && (n0 + BN - 1 > a.gap + w_rmin));
+    need_lim = n0 + BN - 1 > w_limmin;
+    need_doc = false;
     if (DOC) {
-      const IdSummary ks = ksum[cur];
-      skip = skip || !doc_may_keep(w_lo, w_hi, w_glob, ks.lo, ks.hi);
-      need_mask = need_mask || !doc_all_keep(w_lo, w_hi, ks.lo, ks.hi);
+      skip = skip || !doc_may_keep(w_lo, w_hi, w_glob, k_lo, k_hi);
+      need_doc = !doc_all_keep(w_lo, w_hi, k_lo, k_hi);
     }
   }
 };
+
+// Element masks of one 32-key block held in the transposed-score layout: register 4*q4 + t of a
+// lane is key 8*q4 + 4*(lane >> 5) + t of the block.  Both are called under wave-uniform branches.
+//   rel  : (last key the lane's row may see) - (first key of the block) - 4*(lane >> 5)
+FA_DEV void mask_lim(f32x16& s, int rel, float fill) {
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (8 * q4 + t <= rel) ? s[4 * q4 + t] : fill;
+}
+//   ids  : LDS copy of the block's 32 key ids, already offset by 16*(lane >> 5) bytes
+FA_DEV void mask_doc(f32x16& s, const char* ids, int eq_i, bool glob_i, float fill) {
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) {
+    const i32x4 ekv = *reinterpret_cast<const i32x4*>(ids + 32 * q4);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (glob_i || ekv[t] == eq_i) ? s[4 * q4 + t] : fill;
+  }
+}
 
 // ---------------------------------------------------------------------------
 // Work assignment of one workgroup of the forward / dq kernels, including the split of the
