@@ -64,6 +64,9 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) frag[ks] = *reinterpret_cast<const vec8*>(srcp + ks * 16 + g * 8);
   const float c = a.scale_log2e;
+  // rows that may see this lane's key: [row_lo, row_lo + row_span)
+  const int row_lo = CAUSAL ? max(0, key - a.gap) : 0;
+  const unsigned row_span = key < a.N ? (unsigned)(a.M - row_lo) : 0u;
 
   // per query head state (set at the top of the head loop)
   const float* lsep = nullptr;
@@ -130,7 +133,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // One query tile.  BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
     const char* lqt = smem + BUF * TILE_BYTES;
     const char* ldo = smem + (2 + BUF) * TILE_BYTES;
     const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
@@ -138,17 +141,9 @@ void bwd_dkdv_kernel(const KArgs a) {
     const char* t2 = role == 0 ? ldo : lqt;   // transposed operand of the second product
     const int m0 = cur * BQ;  // natural order only
 
-    // wave-level decisions (identical for the two waves of a pair): the tile's 64 rows against keys nw..nw+31
-    bool skip, need_mask;
-    if (!DOC) {
-      skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
-      need_mask = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
-    } else {
-      const IdSummary qs = qsum[cur];
-      skip = (nw >= a.N) || (CAUSAL && (a.gap + qs.rmax < nw)) || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
-      need_mask = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31)) ||
-                  !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
-    }
+    // wave-level decisions (identical for the two waves of a pair), taken by the tile iterator
+    const bool skip = (flags & TF_SKIP) != 0;
+    const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0, has_glob = (flags & TF_GLOB) != 0;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       char* pbuf = smem + P_OFF + (qb * 4 + kb) * P_BYTES + lane * 16;
@@ -169,22 +164,31 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
           }
-          if (need_mask) {
+          if (need_lim) {
+            // row index inside [first row that may see this key, M); padding rows are -1
             asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
               const int i0 = 32 * qb + 8 * q4 + 4 * g;
-              i32x4 eqv = {0, 0, 0, 0};
               i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
-              if (DOC) {
-                eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
-                rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
-              }
+              if (DOC) rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
 #pragma unroll
-              for (int t = 0; t < 4; ++t) {
-                const int i = rowv[t];
-                const bool keep = (i >= 0) && (i < a.M) && keep_elem<CAUSAL, DOC>(i, key, a.gap, a.N, eqv[t], ek_j);
-                x[4 * q4 + t] = keep ? x[4 * q4 + t] : 0.f;
+              for (int t = 0; t < 4; ++t)
+                x[4 * q4 + t] = (unsigned)(rowv[t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
+            }
+          }
+          if (DOC && need_doc) {
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+              const int i0 = 32 * qb + 8 * q4 + 4 * g;
+              const i32x4 eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+              if (!has_glob) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) x[4 * q4 + t] = eqv[t] == ek_j ? x[4 * q4 + t] : 0.f;
+              } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) x[4 * q4 + t] = (eqv[t] >= 0 || eqv[t] == ek_j) ? x[4 * q4 + t] : 0.f;
               }
             }
           }
@@ -261,35 +265,53 @@ void bwd_dkdv_kernel(const KArgs a) {
       nQtiles = a.nQs;
       first = 0;
     }
+    // decisions of this wave pair (keys nw .. nw+31) for query tile t, evaluated by the lane that tests the tile
+    auto dec = [&](int t, const IdSummary& qs) {
+      bool skip, lim, doc = false, glob = false;
+      if (!DOC) {
+        const int m0 = t * BQ;
+        skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
+        lim = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
+      } else {
+        skip = (nw >= a.N) || (CAUSAL && (a.gap + qs.rmax < nw)) || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
+        lim = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31));
+        doc = !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
+        glob = qs.glob != 0;
+      }
+      return (skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0);
+    };
     TileIter it;
-    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000);
+    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000, dec);
     if (gi > 0) __syncthreads();  // the previous head's last tile may still be read from LDS
 
     // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and
     // the row indices of the tile after that are fetched
-    int cur = it.next();
-    int nxt = cur >= 0 ? it.next() : -1;
+    int cur = it.next(dec), cur_fl = it.flags;
+    int nxt = -1, nxt_fl = 0;
+    if (cur >= 0) { nxt = it.next(dec); nxt_fl = it.flags; }
     if (cur >= 0) {
       if (DOC) fetch_idx(cur);
       load_tile(cur, 0);
       if (DOC && nxt >= 0) fetch_idx(nxt);
     }
     while (cur >= 0) {
-      int nxt2 = nxt >= 0 ? it.next() : -1;
+      int nxt2 = -1, nxt2_fl = 0;
+      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; }
       wait_async_loads();
       __syncthreads();
       if (nxt >= 0) load_tile(nxt, 1);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-      compute(0, cur);
-      cur = nxt; nxt = nxt2;
+      compute(0, cur, cur_fl);
+      cur = nxt; cur_fl = nxt_fl; nxt = nxt2; nxt_fl = nxt2_fl;
       if (cur < 0) break;
-      nxt2 = nxt >= 0 ? it.next() : -1;
+      nxt2 = -1;
+      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; }
       wait_async_loads();
       __syncthreads();
       if (nxt >= 0) load_tile(nxt, 0);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-      compute(1, cur);
-      cur = nxt; nxt = nxt2;
+      compute(1, cur, cur_fl);
+      cur = nxt; cur_fl = nxt_fl; nxt = nxt2; nxt_fl = nxt2_fl;
     }
   }
 

@@ -62,8 +62,10 @@ void bwd_dq_kernel(const KArgs a) {
   if (L_i == -INFINITY) L_i = INFINITY;  // row without any kept key: P = exp2(-inf) = 0
   const float delta_i = delp[rowc];
 
+  // decisions of this wave for key tile t, evaluated by the lane that tests the tile
+  auto dec = [&](int t, const IdSummary& ks) { return qc.decide(a, t * BN, BN, ks.lo, ks.hi); };
   TileIter it;
-  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
@@ -77,14 +79,13 @@ void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-  auto compute = [&](const int BUF, const int cur, const int k_lo, const int k_hi) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
     const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
     const int n0 = cur * BN;
-    bool skip, need_lim, need_doc;
-    qc.decide(a, n0, BN, k_lo, k_hi, skip, need_lim, need_doc);
-    if (skip) return;
+    if (flags & TF_SKIP) return;
+    const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -139,23 +140,23 @@ void bwd_dq_kernel(const KArgs a) {
     ldV.issue(t * BN, smem + (2 + BUF) * TILE_BYTES);
     if (DOC && wave == 0) glb_load_lds4(ekp + t * BN + lane, smem + 4 * TILE_BYTES + BUF * (BN * 4));
   };
-  int cur = it.next();
-  int cur_lo = it.t_lo, cur_hi = it.t_hi;
+  int cur = it.next(dec);
+  int cur_fl = it.flags;
   if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
-    int nxt = it.next();
+    int nxt = it.next(dec);
     wait_async_loads();
     __syncthreads();
     if (nxt >= 0) issue(1, nxt);
-    compute(0, cur, cur_lo, cur_hi);
-    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
+    compute(0, cur, cur_fl);
+    cur = nxt; cur_fl = it.flags;
     if (cur < 0) break;
-    nxt = it.next();
+    nxt = it.next(dec);
     wait_async_loads();
     __syncthreads();
     if (nxt >= 0) issue(0, nxt);
-    compute(1, cur, cur_lo, cur_hi);
-    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
+    compute(1, cur, cur_fl);
+    cur = nxt; cur_fl = it.flags;
   }
 
   if (DOC && nsplit > 1) {

@@ -75,8 +75,10 @@ void fwd_kernel(const KArgs a) {
     for (int ks = 0; ks < KS; ++ks) qf[ks] = neg8<E>(qf[ks]);
   }
 
+  // decisions of this wave for key tile t, evaluated by the lane that tests the tile
+  auto dec = [&](int t, const IdSummary& ks) { return qc.decide(a, t * BN, BN, ks.lo, ks.hi); };
   TileIter it;
-  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob);
+  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);
@@ -93,15 +95,14 @@ void fwd_kernel(const KArgs a) {
   float l_run = 0.f;        // this lane's partial row sum
 
   // One K/V tile; BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur, const int k_lo, const int k_hi) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
     const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
     const int n0 = cur * BN;
 
-    bool skip, need_lim, need_doc;
-    qc.decide(a, n0, BN, k_lo, k_hi, skip, need_lim, need_doc);
-    if (skip) return;
+    if (flags & TF_SKIP) return;
+    const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0;
 
     f32x16 s[2];
     __builtin_amdgcn_sched_barrier(0);
@@ -214,23 +215,23 @@ void fwd_kernel(const KArgs a) {
     ldV.issue(t * BN, smem + (2 + BUF) * TILE_BYTES);
     if (DOC && wave == 0) glb_load_lds4(ekp + t * BN + lane, smem + 4 * TILE_BYTES + BUF * (BN * 4));
   };
-  int cur = it.next();
-  int cur_lo = it.t_lo, cur_hi = it.t_hi;
+  int cur = it.next(dec);
+  int cur_fl = it.flags;
   if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
-    int nxt = it.next();
+    int nxt = it.next(dec);
     wait_async_loads();
     __syncthreads();
     if (nxt >= 0) issue(1, nxt);
-    compute(0, cur, cur_lo, cur_hi);
-    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
+    compute(0, cur, cur_fl);
+    cur = nxt; cur_fl = it.flags;
     if (cur < 0) break;
-    nxt = it.next();
+    nxt = it.next(dec);
     wait_async_loads();
     __syncthreads();
     if (nxt >= 0) issue(0, nxt);
-    compute(1, cur, cur_lo, cur_hi);
-    cur = nxt; cur_lo = it.t_lo; cur_hi = it.t_hi;
+    compute(1, cur, cur_fl);
+    cur = nxt; cur_fl = it.flags;
   }
 
   const float l_tot = xhalf_sum(l_run);

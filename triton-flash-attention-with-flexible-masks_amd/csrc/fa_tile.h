@@ -159,53 +159,66 @@ FA_DEV typename E::vec8 lds_tr8(const char* p0, const char* p1) {
 //                 causal mask, its largest row index reaches the own keys
 // With sum == nullptr (no document ids) every tile of the range is visited.
 // ---------------------------------------------------------------------------
+// Wave-level decisions for one tile, taken when the candidates are tested (dec(tile, summary) is
+// evaluated by the lane that tests the tile) and handed out with the tile index, so that the tile
+// loop itself reads nothing from global memory.
+enum { TF_SKIP = 1, TF_LIM = 2, TF_DOC = 4, TF_GLOB = 8 };
+
 struct TileIter {
   unsigned long long mask;
+  unsigned long long fm[4];   // per candidate: the four TF_ bits of dec()
   int base, last;
-  int c_lo, c_hi;          // this lane's candidate (tile base + lane): its id range
-  int t_lo, t_hi;          // id range of the tile returned by the last next() (keys mode, with ids)
+  int flags;                  // TF_ bits of the tile returned by the last next()
   int o_lo, o_hi, o_glob;
   int min_rmax;            // query mode: candidates need rmax >= min_rmax
   bool keys_mode;
   const IdSummary* sum;
 
-  FA_DEV void init_keys(int first, int last_, const IdSummary* ksum, int q_lo, int q_hi, int q_glob) {
+  template <class Dec>
+  FA_DEV void init_keys(int first, int last_, const IdSummary* ksum, int q_lo, int q_hi, int q_glob, const Dec& dec) {
     sum = ksum; o_lo = q_lo; o_hi = q_hi; o_glob = q_glob; keys_mode = true; min_rmax = 0;
-    start(first, last_);
+    start(first, last_, dec);
   }
-  FA_DEV void init_queries(int first, int last_, const IdSummary* qsum, int k_lo, int k_hi, int min_rmax_) {
+  template <class Dec>
+  FA_DEV void init_queries(int first, int last_, const IdSummary* qsum, int k_lo, int k_hi, int min_rmax_, const Dec& dec) {
     sum = qsum; o_lo = k_lo; o_hi = k_hi; o_glob = 0; keys_mode = false; min_rmax = min_rmax_;
-    start(first, last_);
+    start(first, last_, dec);
   }
-  FA_DEV void start(int first, int last_) {
-    last = last_; c_lo = 0; c_hi = -1; t_lo = 0; t_hi = -1;
+  template <class Dec>
+  FA_DEV void start(int first, int last_, const Dec& dec) {
+    last = last_; flags = 0;
     base = (first / 64) * 64;
-    mask = chunk_mask(base) & (~0ull << (first - base));
+    mask = chunk_mask(base, dec) & (~0ull << (first - base));
   }
-  FA_DEV unsigned long long chunk_mask(int b) {
+  template <class Dec>
+  FA_DEV unsigned long long chunk_mask(int b, const Dec& dec) {
     const int t = b + (threadIdx.x & 63);
     bool v = t < last;
+    IdSummary s;
+    s.lo = 0; s.hi = -1; s.glob = 0; s.rmin = 0; s.rmax = -1; s.nvalid = 0; s.kfirst = 0; s.klast = 0;
     if (sum != nullptr && v) {
-      const IdSummary s = sum[t];
-      c_lo = s.lo; c_hi = s.hi;
+      s = sum[t];
       v = keys_mode ? doc_may_keep(o_lo, o_hi, o_glob, s.lo, s.hi)
                     : (s.nvalid > 0 && s.rmax >= min_rmax && doc_may_keep(s.lo, s.hi, s.glob, o_lo, o_hi));
     }
+    const int f = dec(t, s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fm[i] = __builtin_amdgcn_ballot_w64(((f >> i) & 1) != 0);
     return __builtin_amdgcn_ballot_w64(v);
   }
   // next tile index, or -1
-  FA_DEV int next() {
+  template <class Dec>
+  FA_DEV int next(const Dec& dec) {
     while (mask == 0) {
       base += 64;
       if (base >= last) return -1;
-      mask = chunk_mask(base);
+      mask = chunk_mask(base, dec);
     }
     const int jl = __builtin_ctzll(mask);
     mask &= mask - 1;
-    if (sum != nullptr) {   // no memory access in the tile loop: the range comes out of the registers
-      t_lo = __builtin_amdgcn_readlane(c_lo, jl);
-      t_hi = __builtin_amdgcn_readlane(c_hi, jl);
-    }
+    flags = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) flags |= int((fm[i] >> jl) & 1) << i;
     return base + jl;
   }
 };
@@ -286,18 +299,19 @@ struct QTileCtx {
     return min((hi_key + 63) / 64, g_klast + 1);
   }
 
-  // Wave-level decisions for the key tile n0 .. n0+BN-1 whose ids span [k_lo, k_hi]:
-  //   skip     : no (row, key) pair of the wave's rows is kept
-  //   need_lim : some pair fails the causal / length limit  -> mask_lim
-  //   need_doc : some pair may fail the id test             -> mask_doc
-  FA_DEV void decide(const KArgs& a, int n0, int BN, int k_lo, int k_hi, bool& skip, bool& need_lim, bool& need_doc) const {
-    skip = (w_rmax < 0) || (CAUSAL && (n0 > a.gap + w_rmax));
-    need_lim = n0 + BN - 1 > w_limmin;
-    need_doc = false;
+  // Wave-level decisions (TF_ bits) for the key tile n0 .. n0+BN-1 whose ids span [k_lo, k_hi]:
+  //   TF_SKIP : no (row, key) pair of the wave's rows is kept
+  //   TF_LIM  : some pair fails the causal / length limit  -> mask_lim
+  //   TF_DOC  : some pair may fail the id test             -> mask_doc
+  FA_DEV int decide(const KArgs& a, int n0, int BN, int k_lo, int k_hi) const {
+    bool skip = (w_rmax < 0) || (CAUSAL && (n0 > a.gap + w_rmax));
+    const bool need_lim = n0 + BN - 1 > w_limmin;
+    bool need_doc = false;
     if (DOC) {
       skip = skip || !doc_may_keep(w_lo, w_hi, w_glob, k_lo, k_hi);
       need_doc = !doc_all_keep(w_lo, w_hi, k_lo, k_hi);
     }
+    return (skip ? TF_SKIP : 0) | (need_lim ? TF_LIM : 0) | (need_doc ? TF_DOC : 0);
   }
 };
 
