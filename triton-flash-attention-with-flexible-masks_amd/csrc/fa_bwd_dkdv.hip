@@ -63,6 +63,8 @@ void bwd_dkdv_kernel(const KArgs a) {
   vec8 frag[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) frag[ks] = *reinterpret_cast<const vec8*>(srcp + ks * 16 + g * 8);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) settle(frag[ks]);
   const float c = a.scale_log2e;
   // rows that may see this lane's key: [row_lo, row_lo + row_span)
   const int row_lo = CAUSAL ? max(0, key - a.gap) : 0;

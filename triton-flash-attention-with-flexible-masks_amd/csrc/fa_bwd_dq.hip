@@ -60,7 +60,11 @@ void bwd_dq_kernel(const KArgs a) {
   const float c = a.scale_log2e;
   float L_i = lsep[rowc];
   if (L_i == -INFINITY) L_i = INFINITY;  // row without any kept key: P = exp2(-inf) = 0
-  const float delta_i = delp[rowc];
+  float delta_i = delp[rowc];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) { settle(qf[ks]); settle(dof[ks]); }
+  settle(L_i);
+  settle(delta_i);
 
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
   auto dec = [&](int t, const IdSummary& ks) { return qc.decide(a, t * BN, BN, ks.lo, ks.hi); };

@@ -116,6 +116,19 @@ FA_DEV float xhalf_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Make a 16-byte value loaded from global memory "used" right here.  The compiler waits for a
+// load at the first use of its result; for operands that are loaded once and first used inside
+// the tile loop that wait (s_waitcnt vmcnt) would sit in the loop, where it also waits for the
+// asynchronous tile loads issued just before it -- the loads it is meant to overlap with.
+template <typename V>
+FA_DEV void settle(V& x) {
+  i32x4 u = __builtin_bit_cast(i32x4, x);
+  asm volatile("" : "+v"(u));
+  x = __builtin_bit_cast(V, u);
+}
+FA_DEV void settle(float& x) { asm volatile("" : "+v"(x)); }
+FA_DEV void settle(int& x) { asm volatile("" : "+v"(x)); }
+
 FA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -68,6 +68,8 @@ void fwd_kernel(const KArgs a) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
     qf[ks] = *reinterpret_cast<const vec8*>(qp + int64_t(rowc) * a.q_rs + ks * 16 + g * 8);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) settle(qf[ks]);
   float c = a.scale_log2e;
   if (c < 0.f) {  // keep max(raw score) == max(scaled score): move the sign into Q
     c = -c;
