@@ -45,7 +45,12 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled per (workload, kernel); None = not measured.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # bytes per launch: FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (factors from a 1 GiB copy in the same runs)
+    ("cfg4_doc_causal_16k", "fa_bwd_dkdv"): 816_500_000,
+    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_380_000_000,
+    ("cfg4_doc_causal_16k", "fa_fwd"): 1_250_000_000,
+}
 
 
 def parse_args():
@@ -56,6 +61,9 @@ def parse_args():
     ap.add_argument("--workload", default="cfg4_doc_causal_16k")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-heads", type=int, default=2, help="(batch, head) slices timed on the CPU")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch plain device copies of 1 GiB: the reference point that scales "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE readings to bytes")
     return ap.parse_args()
 
 
@@ -170,6 +178,13 @@ def main():
         out = attention(q, k, v, w.causal, scale, eq, ek, mode)
         out.backward(do)
 
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -126,7 +126,11 @@ uint64_t fa_workspace_bytes(const fa_params* p);
 
 /* Mask engine: normalise eq/ek to int32 and build per-tile id summaries
    into p->workspace.  Must be enqueued before fa_fwd / fa_bwd_* on the same
-   stream whenever score_mode != 0.  The same workspace serves forward and backward. */
+   stream whenever score_mode != 0.  The same workspace serves forward and backward.
+   The plan depends on the ids, the sizes AND on `causal` (key ranges are narrowed with the
+   causal bound): plan again when any of them changes.  The workspace also holds the scratch
+   of the tiles whose key range is split over several workgroups, so two launches that share a
+   workspace must be ordered on one stream. */
 int fa_mask_plan(const fa_params* p, void* stream);
 
 /* O = softmax(q k^T * sm_scale + mask) v ; lse = log2-sum-exp2 of the scaled scores. */
