@@ -138,6 +138,39 @@ def test_long_key_ranges_of_global_rows():
     _run_case(2, 2, 2, 2048, 2048, 16, torch.bfloat16, True, True, seed=24)
 
 
+def test_transposed_views_and_strided_gradients():
+    """q, k, v, dO given as [B, L, H, D] storage viewed as [B, H, L, D] (cf. testing.py:59-66): the kernels
+    take element strides, nothing is copied on the way in."""
+    from flash_mi355 import attention, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    B, H, L, D = 2, 3, 320, 64
+    g = torch.Generator().manual_seed(77)
+    rng = np.random.default_rng(77)
+    base = [torch.randn(B, L, H, D, generator=g).bfloat16() for _ in range(4)]
+    q, k, v, do = (t.transpose(1, 2) for t in base)
+    ek = torch.from_numpy(_ids(rng, B, H, L, "uniform"))[:, None, :].expand(B, H, L)
+    print("case transposed views", flush=True)
+    qd, kd, vd = (t.cuda().transpose(1, 2).requires_grad_(True) for t in base[:3])
+    assert not qd.is_contiguous() and qd.stride(-1) == 1
+    out = attention(qd, kd, vd, True, None, ek.cuda(), ek.cuda(), SCORE_FUNC_MODE1_DOC)
+    out.backward(base[3].cuda().transpose(1, 2))
+    ref = O.attention_autograd(q, k, v, do, True, None, ek, ek, 1)
+    for name, got, want in (("o", out, ref[0]), ("dq", qd.grad, ref[2]), ("dk", kd.grad, ref[3]), ("dv", vd.grad, ref[4])):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
+
+
+def test_harness_cell_runs_and_agrees():
+    from flash_mi355 import harness as Hn
+    torch.manual_seed(5)
+    checks, benches = Hn.run_attn(["torch", "mem", "mi355"], [2, 2, 256, 64], True, "bf16", True,
+                                  check_times=1, bench_times=2, warmup_times=1)
+    for key, diffs in checks:
+        if key["func_name"] == "mi355":
+            assert all(0 <= d <= 5e-2 for d in diffs), diffs
+    assert len(benches) == 9 and all(float(b[1][0]) > 0 for b in benches if b[0]["func_name"] == "mi355")
+
+
 def test_per_head_int64_ids():
     _run_case(1, 3, 3, 192, 192, 64, torch.bfloat16, True, True, seed=9, per_head_ids=True, id_dtype=torch.int64)
 
