@@ -10,6 +10,12 @@
 // Same workgroup shape, LDS staging and tile skipping as the forward kernel.
 
 #include "fa_tile.h"
+#ifndef FA_DQ_PRE
+#define FA_DQ_PRE 4
+#endif
+#ifndef FA_DQ_PRE2
+#define FA_DQ_PRE2 3
+#endif
 
 namespace fa {
 
@@ -94,16 +100,27 @@ void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       f32x16 s = zero, dp = zero;
+      __builtin_amdgcn_sched_barrier(0);
+      // S and dP are accumulated alternately (an MFMA that accumulates onto the result of the MFMA
+      // issued right before it waits a full extra MFMA time), operands a few LDS reads ahead.
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
         s = E::mfma32(kf, qf[ks], s);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
         const vec8 vf = lds_row8<E>(lv + lo.row[ks] + kb * 32 * DL * 2);
         dp = E::mfma32(vf, dof[ks], dp);
       }
+      {
+        constexpr int NM = 2 * KS, PRE = NM < FA_DQ_PRE ? NM : FA_DQ_PRE;
+        __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+        for (int i = 0; i < NM - PRE; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
       // P and dS for this lane's 16 keys of the block
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -118,6 +135,7 @@ void bwd_dq_kernel(const KArgs a) {
         asm volatile("" ::: "memory");
         mask_doc(s, lid + kb * 32 * 4, eq_i, qc.glob_i, 0.f);
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         vec8 dsf;
@@ -134,6 +152,18 @@ void bwd_dq_kernel(const KArgs a) {
           dq[db] = E::mfma32(ktf, dsf, dq[db]);
         }
       }
+      // K^T fragments (two transposed reads each) a few MFMAs ahead; dS conversions just in time
+      {
+        constexpr int NM = 2 * DBN, PRE = NM < FA_DQ_PRE2 ? NM : FA_DQ_PRE2;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+          if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
