@@ -341,12 +341,8 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   const int slots = (a.B * a.Hk + 7) / 8;
   const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + 8 * 4096;
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static bool lds_allowed[64] = {};   // per kernel instantiation and device
+  if (int e = allow_lds(kern, lds, lds_allowed)) return e;
   hipLaunchKernelGGL(kern, dim3(8 * slots * nKt), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }

@@ -33,6 +33,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 #define FA_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define FA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 #define FA_DEV __device__ __forceinline__
+#define FA_HD __host__ __device__ inline
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -261,6 +262,21 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_sk_o = take(nsk * kSplitK * 128 * uint64_t(p->D) * 4);
   w.total = o;
   return w;
+}
+
+// Raise the dynamic LDS limit of a kernel once per device (the attribute is per device and per
+// kernel; a process may drive several GPUs).  `done` is the caller's per-kernel record.
+template <typename K>
+static int allow_lds(K kern, size_t lds, bool (&done)[64]) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64 || !done[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    if (dev >= 0 && dev < 64) done[dev] = true;
+  }
+  return 0;
 }
 
 // Launchers implemented one per translation unit; each returns a hipError_t as int.

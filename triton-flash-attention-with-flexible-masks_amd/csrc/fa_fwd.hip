@@ -43,7 +43,7 @@ void fwd_kernel(const KArgs a) {
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
   // order and see the longest key ranges; without ids the last rows do
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
-  const int nSlots = nQt + (DOC ? kSplitExtra : 0);
+  const int nSlots = nQt + (DOC ? split_extra(a.nKs) : 0);
   int slot, bh;
   if (!block_to_tile(nSlots, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
@@ -312,16 +312,12 @@ void fwd_kernel(const KArgs a) {
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
-  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? kSplitExtra : 0);
+  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? split_extra(a.nKs) : 0);
   const int slots = (a.B * a.H + 7) / 8;
   const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2 + 2 * BN * 4;  // K, V double buffered + key ids
   auto kern = fwd_kernel<Tag, D, CAUSAL, DOC>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static bool lds_allowed[64] = {};   // per kernel instantiation and device
+  if (int e = allow_lds(kern, lds, lds_allowed)) return e;
   hipLaunchKernelGGL(kern, dim3(8 * slots * nQt), dim3(256), lds, s, a);
   return (int)hipGetLastError();
 }

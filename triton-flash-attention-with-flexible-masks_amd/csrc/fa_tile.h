@@ -345,20 +345,23 @@ struct QWork {
   int gt;      // index among the splittable global-row tiles, or -1
   int split;   // chunk of the key range handled by this workgroup
 };
-constexpr int kSplitExtra = kSplitTiles * (kSplitK - 1);
+// Extra workgroup slots per (batch, head) for chunks 1 .. kSplitK-1; none when no key range can be
+// long enough to be cut (split_range needs 2 * kSplitMinTiles key tiles): empty workgroups are not free.
+FA_HD int split_extra(int nKs) { return nKs >= 2 * kSplitMinTiles ? kSplitTiles * (kSplitK - 1) : 0; }
 
 template <bool DOC>
 FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
   if (!DOC) { w.tile = nQt - 1 - slot; w.gt = -1; w.split = 0; return true; }
   const QHeader hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
   const int g0 = hd.nLp / 128;   // first global-row tile
-  if (slot < kSplitExtra) {
+  const int nE = split_extra(a.nKs);
+  if (slot < nE) {
     w.gt = slot / (kSplitK - 1);
     w.split = 1 + slot % (kSplitK - 1);
     w.tile = g0 + w.gt;
     return w.tile < hd.nT128;
   }
-  w.tile = nQt - 1 - (slot - kSplitExtra);
+  w.tile = nQt - 1 - (slot - nE);
   w.split = 0;
   w.gt = (w.tile >= g0 && w.tile - g0 < kSplitTiles) ? w.tile - g0 : -1;
   return true;
