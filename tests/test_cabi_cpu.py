@@ -84,8 +84,13 @@ def test_workspace_size():
     r256 = lambda x: (x + 255) // 256 * 256
     Pp = 256 + 256
     want = (r256(128 * 4) + r256(4 * 256 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
-            + r256(4 * 4 * 32)
-            # split global-row tiles: counters, (max, sum) pairs, fp32 partial tiles
+            + r256(4 * 4 * 32))
+    assert L.fa_workspace_bytes(ctypes.byref(p)) == want   # 4 key tiles of 64: no key range is ever split
+    # from 32 key tiles on, scratch for split global-row tiles: counters, (max, sum) pairs, fp32 partial tiles
+    p.N = 2048
+    p.ek_stride[0], p.ek_stride[1] = 4 * 2048, 2048
+    want = (r256(128 * 4) + r256(4 * 2048 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+            + r256(4 * 32 * 32)
             + r256(4 * 8 * 4) + r256(4 * 8 * 4 * 128 * 2 * 4) + r256(4 * 8 * 4 * 128 * p.D * 4))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want
 

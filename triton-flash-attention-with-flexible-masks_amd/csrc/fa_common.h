@@ -181,6 +181,10 @@ FA_DEV bool doc_all_keep(int q_lo, int q_hi, int k_lo, int k_hi) {
   return (q_lo > q_hi) || (q_lo == q_hi && k_lo == k_hi && q_lo == k_lo);
 }
 
+// Extra workgroup slots per (batch, head) for chunks 1 .. kSplitK-1; none when no key range can be
+// long enough to be cut (split_range needs 2 * kSplitMinTiles key tiles): empty workgroups are not free.
+FA_HD int split_extra(int nKs) { return nKs >= 2 * kSplitMinTiles ? kSplitTiles * (kSplitK - 1) : 0; }
+
 // Kernel-side view of the operands (built on the host from fa_params).
 struct KArgs {
   const void* q;
@@ -256,7 +260,8 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_qhdr = take(uint64_t(p->B) * w.Hq1 * sizeof(QHeader));
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
-  const uint64_t nsk = uint64_t(p->B) * p->H * kSplitTiles;
+  // scratch of the split tiles: only when a key range can be long enough to be cut
+  const uint64_t nsk = split_extra(w.nKs) > 0 ? uint64_t(p->B) * p->H * kSplitTiles : 0;
   w.off_sk_cnt = take(nsk * 4);
   w.off_sk_ml = take(nsk * kSplitK * 128 * 2 * 4);
   w.off_sk_o = take(nsk * kSplitK * 128 * uint64_t(p->D) * 4);

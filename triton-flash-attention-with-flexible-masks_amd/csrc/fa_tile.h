@@ -345,9 +345,6 @@ struct QWork {
   int gt;      // index among the splittable global-row tiles, or -1
   int split;   // chunk of the key range handled by this workgroup
 };
-// Extra workgroup slots per (batch, head) for chunks 1 .. kSplitK-1; none when no key range can be
-// long enough to be cut (split_range needs 2 * kSplitMinTiles key tiles): empty workgroups are not free.
-FA_HD int split_extra(int nKs) { return nKs >= 2 * kSplitMinTiles ? kSplitTiles * (kSplitK - 1) : 0; }
 
 template <bool DOC>
 FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
