@@ -119,8 +119,7 @@ class FlashAttention(torch.autograd.Function):
         assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
         if score_func_mode != SCORE_FUNC_MODE0_NOPE:
             eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
-            assert eq.dtype == ek.dtype or True
-            if eq.dtype != ek.dtype:
+            if eq.dtype != ek.dtype:   # one id width per call
                 eq, ek = eq.to(torch.int64), ek.to(torch.int64)
             assert tuple(eq.shape) == (B, H, M), "eq must be [bs, H, Lq]"
             assert tuple(ek.shape) == (B, H, N), "ek must be [bs, H, Lk]"
