@@ -135,7 +135,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // One query tile.  BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
+  auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
     const char* lqt = smem + BUF * TILE_BYTES;
     const char* ldo = smem + (2 + BUF) * TILE_BYTES;
     const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
@@ -178,6 +178,14 @@ void bwd_dkdv_kernel(const KArgs a) {
               for (int t = 0; t < 4; ++t)
                 x[4 * q4 + t] = (unsigned)(rowv[t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
             }
+          }
+          if (DOC && (flags & TF_COL)) {
+            // every row of the tile carries the same local id: the id test depends on the key alone,
+            // i.e. on the lane -- whole columns of the block are kept or dropped
+            asm volatile("" ::: "memory");
+            const bool col_keep = ek_j == tile_id;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) x[r] = col_keep ? x[r] : 0.f;
           }
           if (DOC && need_doc) {
             asm volatile("" ::: "memory");
@@ -269,7 +277,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
     // decisions of this wave pair (keys nw .. nw+31) for query tile t, evaluated by the lane that tests the tile
     auto dec = [&](int t, const IdSummary& qs) {
-      bool skip, lim, doc = false, glob = false;
+      bool skip, lim, doc = false, glob = false, col = false;
       if (!DOC) {
         const int m0 = t * BQ;
         skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
@@ -279,8 +287,12 @@ void bwd_dkdv_kernel(const KArgs a) {
         lim = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31));
         doc = !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
         glob = qs.glob != 0;
+        // one local id for the whole tile (padding rows aside, which the row-range mask drops):
+        // the cheap column form of the id mask replaces the element form
+        col = doc && !glob && qs.lo == qs.hi;
+        if (col) doc = false;
       }
-      return (skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0);
+      return tile_value((skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0) | (col ? TF_COL : 0), qs.lo);
     };
     TileIter it;
     it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000, dec);
@@ -288,32 +300,32 @@ void bwd_dkdv_kernel(const KArgs a) {
 
     // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and
     // the row indices of the tile after that are fetched
-    int cur = it.next(dec), cur_fl = it.flags;
-    int nxt = -1, nxt_fl = 0;
-    if (cur >= 0) { nxt = it.next(dec); nxt_fl = it.flags; }
+    int cur = it.next(dec), cur_fl = it.flags, cur_id = it.value;
+    int nxt = -1, nxt_fl = 0, nxt_id = 0;
+    if (cur >= 0) { nxt = it.next(dec); nxt_fl = it.flags; nxt_id = it.value; }
     if (cur >= 0) {
       if (DOC) fetch_idx(cur);
       load_tile(cur, 0);
       if (DOC && nxt >= 0) fetch_idx(nxt);
     }
     while (cur >= 0) {
-      int nxt2 = -1, nxt2_fl = 0;
-      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; }
+      int nxt2 = -1, nxt2_fl = 0, nxt2_id = 0;
+      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; nxt2_id = it.value; }
       wait_async_loads();
       __syncthreads();
       if (nxt >= 0) load_tile(nxt, 1);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-      compute(0, cur, cur_fl);
-      cur = nxt; cur_fl = nxt_fl; nxt = nxt2; nxt_fl = nxt2_fl;
+      compute(0, cur, cur_fl, cur_id);
+      cur = nxt; cur_fl = nxt_fl; cur_id = nxt_id; nxt = nxt2; nxt_fl = nxt2_fl; nxt_id = nxt2_id;
       if (cur < 0) break;
       nxt2 = -1;
-      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; }
+      if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; nxt2_id = it.value; }
       wait_async_loads();
       __syncthreads();
       if (nxt >= 0) load_tile(nxt, 0);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
-      compute(1, cur, cur_fl);
-      cur = nxt; cur_fl = nxt_fl; nxt = nxt2; nxt_fl = nxt2_fl;
+      compute(1, cur, cur_fl, cur_id);
+      cur = nxt; cur_fl = nxt_fl; cur_id = nxt_id; nxt = nxt2; nxt_fl = nxt2_fl; nxt_id = nxt2_id;
     }
   }
 

@@ -78,7 +78,7 @@ void fwd_kernel(const KArgs a) {
   }
 
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
-  auto dec = [&](int t, const IdSummary& ks) { return qc.decide(a, t * BN, BN, ks.lo, ks.hi); };
+  auto dec = [&](int t, const IdSummary& ks) { return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi), 0); };
   TileIter it;
   it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);
 

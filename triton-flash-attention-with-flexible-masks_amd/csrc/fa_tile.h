@@ -162,11 +162,16 @@ FA_DEV typename E::vec8 lds_tr8(const char* p0, const char* p1) {
 // Wave-level decisions for one tile, taken when the candidates are tested (dec(tile, summary) is
 // evaluated by the lane that tests the tile) and handed out with the tile index, so that the tile
 // loop itself reads nothing from global memory.
-enum { TF_SKIP = 1, TF_LIM = 2, TF_DOC = 4, TF_GLOB = 8 };
+// dec() returns the TF_ bits in its low word and, optionally, one value in its high word
+// (tile_value(): handed out as `value`, e.g. the single id of a tile).
+enum { TF_SKIP = 1, TF_LIM = 2, TF_DOC = 4, TF_GLOB = 8, TF_COL = 16, TF_NBITS = 5 };
+FA_DEV long long tile_value(int flags, int value) { return (long long)(unsigned)flags | ((long long)value << 32); }
 
 struct TileIter {
   unsigned long long mask;
-  unsigned long long fm[4];   // per candidate: the four TF_ bits of dec()
+  unsigned long long fm[TF_NBITS];   // per candidate: the TF_ bits of dec()
+  int c_val;                  // per lane: the value dec() attached to this lane's candidate
+  int value;                  // that value for the tile returned by the last next()
   int base, last;
   int flags;                  // TF_ bits of the tile returned by the last next()
   int o_lo, o_hi, o_glob;
@@ -186,7 +191,7 @@ struct TileIter {
   }
   template <class Dec>
   FA_DEV void start(int first, int last_, const Dec& dec) {
-    last = last_; flags = 0;
+    last = last_; flags = 0; c_val = 0; value = 0;
     base = (first / 64) * 64;
     mask = chunk_mask(base, dec) & (~0ull << (first - base));
   }
@@ -201,9 +206,11 @@ struct TileIter {
       v = keys_mode ? doc_may_keep(o_lo, o_hi, o_glob, s.lo, s.hi)
                     : (s.nvalid > 0 && s.rmax >= min_rmax && doc_may_keep(s.lo, s.hi, s.glob, o_lo, o_hi));
     }
-    const int f = dec(t, s);
+    const long long fv = dec(t, s);
+    const int f = (int)fv;
+    c_val = (int)(fv >> 32);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fm[i] = __builtin_amdgcn_ballot_w64(((f >> i) & 1) != 0);
+    for (int i = 0; i < TF_NBITS; ++i) fm[i] = __builtin_amdgcn_ballot_w64(((f >> i) & 1) != 0);
     return __builtin_amdgcn_ballot_w64(v);
   }
   // next tile index, or -1
@@ -218,7 +225,8 @@ struct TileIter {
     mask &= mask - 1;
     flags = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) flags |= int((fm[i] >> jl) & 1) << i;
+    for (int i = 0; i < TF_NBITS; ++i) flags |= int((fm[i] >> jl) & 1) << i;
+    value = __builtin_amdgcn_readlane(c_val, jl);
     return base + jl;
   }
 };
