@@ -21,6 +21,12 @@
 // are visited.  The query heads of a grouped-query group are walked inside the kernel, so dK, dV
 // are written once, already summed (the reference sums afterwards, flash_triton.py:635-637).
 #include "fa_tile.h"
+#ifndef FA_KV_PRE
+#define FA_KV_PRE 4
+#endif
+#ifndef FA_KV_PRE2
+#define FA_KV_PRE2 3
+#endif
 
 namespace fa {
 
@@ -151,12 +157,24 @@ void bwd_dkdv_kernel(const KArgs a) {
       char* pbuf = smem + P_OFF + (qb * 4 + kb) * P_BYTES + lane * 16;
       f32x16 x = zero;
       if (!skip) {
-        // first product: S (score wave) or dP (gradient wave)
+        // first product: S (score wave) or dP (gradient wave); operand rows a few LDS reads ahead
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const vec8 ra = lds_row8<E>(t1 + lo.row[ks] + qb * 32 * DL * 2);
           x = E::mfma32(ra, frag[ks], x);
         }
+        {
+          constexpr int PRE = KS < FA_KV_PRE ? KS : FA_KV_PRE;
+          __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+          for (int i = 0; i < KS - PRE; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (role == 0) {
           // S -> P for this lane's 16 query rows of the block
 #pragma unroll
@@ -224,6 +242,7 @@ void bwd_dkdv_kernel(const KArgs a) {
           }
         }
         // second product: dV^T += dO^T P (score wave) or dK^T += Q^T dS (gradient wave)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           vec8 yf;
@@ -239,6 +258,18 @@ void bwd_dkdv_kernel(const KArgs a) {
             acc[db] = E::mfma32(tf, yf, acc[db]);
           }
         }
+        // transposed fragments (two reads each) a few MFMAs ahead, conversions just in time
+        {
+          constexpr int NM = 2 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
+#pragma unroll
+          for (int i = 0; i < NM; ++i) {
+            if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
