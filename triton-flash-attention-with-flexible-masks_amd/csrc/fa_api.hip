@@ -98,6 +98,7 @@ static KArgs make_args(const fa_params* p) {
   a.scale_log2e = p->sm_scale * kLog2e;
   a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.peq = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;
   a.sk_cnt = nullptr; a.sk_ml = nullptr; a.sk_o = nullptr;
+  a.split_k = 1; a.split_tiles = 0;
   a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.pm_bs = a.pm_hs = a.qh_bs = a.qh_hs = 0;
   a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
   a.nQs = a.nKs = a.Pp = 0;
@@ -118,6 +119,8 @@ static KArgs make_args(const fa_params* p) {
     a.qs_bs = int64_t(w.Hq1) * w.nQs; a.qs_hs = w.Hq1 == 1 ? 0 : w.nQs;
     a.ks_bs = int64_t(w.Hk1) * w.nKs; a.ks_hs = w.Hk1 == 1 ? 0 : w.nKs;
     a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
+    const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
+    a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);
     a.sk_ml = reinterpret_cast<float*>(ws + w.off_sk_ml);
     a.sk_o = reinterpret_cast<float*>(ws + w.off_sk_o);

@@ -381,12 +381,11 @@ template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BK = 128, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const int slots = (a.B * a.Hk + 7) / 8;
   const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + 8 * 4096;
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
-  hipLaunchKernelGGL(kern, dim3(8 * slots * nKt), dim3(512), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 

@@ -44,12 +44,27 @@ constexpr int kSumRows = 64;
 constexpr int kPermAlign = 256;
 // Tiles of global rows (eq >= 0) see every key up to their own position, i.e. up to the whole
 // sequence: a single workgroup walking 16K keys is the critical path of the kernel.  The key range
-// of the first kSplitTiles such tiles of a (batch, head) is therefore cut into up to kSplitK chunks
-// handled by different workgroups; each writes an fp32 partial result and the last one to arrive
-// (an atomic counter per tile) merges them.  The merge order is fixed, results stay reproducible.
-constexpr int kSplitK = 4;
-constexpr int kSplitTiles = 8;
+// of the first `tiles` such tiles of a (batch, head) is therefore cut into up to `k` chunks handled
+// by different workgroups; each writes an fp32 partial result and the last one to arrive (an atomic
+// counter per tile) merges them.  The merge order is fixed, results stay reproducible.
 constexpr int kSplitMinTiles = 16;   // key tiles (of 64) per chunk below which splitting does not pay
+constexpr int kSplitKMax = 4;        // more chunks did not pay on any measured shape
+struct SplitCfg {
+  int k;      // chunks per tile (1: nothing is ever split)
+  int tiles;  // global-row tiles per (batch, head) that can be split
+};
+// Chunks of at least 32 key tiles (2 .. kSplitKMax of them), and as many splittable tiles as 128 MB of
+// scratch allow (8 .. 64): long sequences with few heads have many global-row tiles, each of them long.
+inline SplitCfg split_config(int B, int H, int N, int D) {
+  SplitCfg c = {1, 0};
+  const int nKs = (N + kSumRows - 1) / kSumRows;
+  if (nKs < 2 * kSplitMinTiles) return c;   // no key range can be long enough to be cut
+  c.k = nKs / 32 < 2 ? 2 : (nKs / 32 > kSplitKMax ? kSplitKMax : nKs / 32);
+  const uint64_t per_tile = uint64_t(c.k) * 128 * (D + 2) * 4;
+  const uint64_t t = (uint64_t(128) << 20) / (uint64_t(B) * H * per_tile);
+  c.tiles = t < 8 ? 8 : (t > 64 ? 64 : int(t));
+  return c;
+}
 
 struct bf16_t {};
 struct fp16_t {};
@@ -181,10 +196,6 @@ FA_DEV bool doc_all_keep(int q_lo, int q_hi, int k_lo, int k_hi) {
   return (q_lo > q_hi) || (q_lo == q_hi && k_lo == k_hi && q_lo == k_lo);
 }
 
-// Extra workgroup slots per (batch, head) for chunks 1 .. kSplitK-1; none when no key range can be
-// long enough to be cut (split_range needs 2 * kSplitMinTiles key tiles): empty workgroups are not free.
-FA_HD int split_extra(int nKs) { return nKs >= 2 * kSplitMinTiles ? kSplitTiles * (kSplitK - 1) : 0; }
-
 // Kernel-side view of the operands (built on the host from fa_params).
 struct KArgs {
   const void* q;
@@ -204,10 +215,11 @@ struct KArgs {
   const QHeader* qhdr;    // [B, Hq']
   const IdSummary* qsum;  // [B, Hq', nQs]  per 64 entries of the permuted order
   const IdSummary* ksum;  // [B, Hk', nKs]  per 64 keys
-  // split-key scratch of the global-row tiles, see kSplitK: per (b, h, global tile g)
-  int* sk_cnt;            // [B, H, kSplitTiles]              arrival counters (zero between kernels)
-  float* sk_ml;           // [B, H, kSplitTiles, kSplitK, 128, 2]  per row: reference point, row sum
-  float* sk_o;            // [B, H, kSplitTiles, kSplitK, 128, D]  per row: unnormalised partial result
+  // split-key scratch of the global-row tiles, see SplitCfg: per (b, h, global tile g)
+  int split_k, split_tiles;
+  int* sk_cnt;            // [B, H, split_tiles]                  arrival counters (zero between kernels)
+  float* sk_ml;           // [B, H, split_tiles, split_k, 128, 2]  per row: reference point, row sum
+  float* sk_o;            // [B, H, split_tiles, split_k, 128, D]  per row: unnormalised partial result
   int64_t q_bs, q_hs, q_rs;
   int64_t k_bs, k_hs, k_rs;
   int64_t v_bs, v_hs, v_rs;
@@ -261,10 +273,11 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
   // scratch of the split tiles: only when a key range can be long enough to be cut
-  const uint64_t nsk = split_extra(w.nKs) > 0 ? uint64_t(p->B) * p->H * kSplitTiles : 0;
+  const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
+  const uint64_t nsk = uint64_t(p->B) * p->H * sc.tiles;
   w.off_sk_cnt = take(nsk * 4);
-  w.off_sk_ml = take(nsk * kSplitK * 128 * 2 * 4);
-  w.off_sk_o = take(nsk * kSplitK * 128 * uint64_t(p->D) * 4);
+  w.off_sk_ml = take(nsk * sc.k * 128 * 2 * 4);
+  w.off_sk_o = take(nsk * sc.k * 128 * uint64_t(p->D) * 4);
   w.total = o;
   return w;
 }

@@ -43,7 +43,7 @@ void fwd_kernel(const KArgs a) {
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
   // order and see the longest key ranges; without ids the last rows do
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
-  const int nSlots = nQt + (DOC ? split_extra(a.nKs) : 0);
+  const int nSlots = nQt + (DOC ? split_extra(a) : 0);
   int slot, bh;
   if (!block_to_tile(nSlots, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
@@ -52,7 +52,7 @@ void fwd_kernel(const KArgs a) {
   QTileCtx<CAUSAL, DOC> qc;
   if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
   int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
-  const int nsplit = split_range(wk, kt_first, kt_last);
+  const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
@@ -240,9 +240,9 @@ void fwd_kernel(const KArgs a) {
   if (DOC && nsplit > 1) {
     // This workgroup saw one chunk of the keys: store the unnormalised partial result; the last
     // chunk to arrive combines them (log-sum-exp merge) and writes O and LSE.
-    const int64_t tbase = (int64_t(b) * a.H + h) * kSplitTiles + wk.gt;
-    float* po = a.sk_o + (tbase * kSplitK + wk.split) * (128 * D);
-    float* pml = a.sk_ml + (tbase * kSplitK + wk.split) * (128 * 2);
+    const int64_t tbase = (int64_t(b) * a.H + h) * a.split_tiles + wk.gt;
+    float* po = a.sk_o + (tbase * a.split_k + wk.split) * (128 * D);
+    float* pml = a.sk_ml + (tbase * a.split_k + wk.split) * (128 * 2);
     const int rt = (threadIdx.x >> 6) * 32 + (lane & 31);   // row inside the tile
     if (g == 0) store_dev(pml + rt * 2, m_ref, l_tot);
 #pragma unroll
@@ -256,28 +256,26 @@ void fwd_kernel(const KArgs a) {
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
     // merge: the whole workgroup walks the tile, one float4 of one row per thread and step
     constexpr int C4 = D / 4;
-    const float* bo = a.sk_o + tbase * kSplitK * (128 * D);
-    const float* bml = a.sk_ml + tbase * kSplitK * (128 * 2);
+    const float* bo = a.sk_o + tbase * a.split_k * (128 * D);
+    const float* bml = a.sk_ml + tbase * a.split_k * (128 * 2);
     const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
       const int r = i / C4, c = i % C4;
       const int mrow = prm[r];
       if (mrow < 0) continue;
-      float ms[kSplitK], ls[kSplitK], mmax = -INFINITY;
-#pragma unroll
-      for (int sp = 0; sp < kSplitK; ++sp) {
-        const bool on = sp < nsplit;
-        ms[sp] = -INFINITY; ls[sp] = 0.f;
-        if (on) load_dev(bml + sp * 256 + r * 2, ms[sp], ls[sp]);
-        mmax = fmaxf(mmax, ms[sp]);
+      float mmax = -INFINITY;
+      for (int sp = 0; sp < nsplit; ++sp) {
+        float m_, l_;
+        load_dev(bml + sp * 256 + r * 2, m_, l_);
+        mmax = fmaxf(mmax, m_);
       }
       float lsum = 0.f;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int sp = 0; sp < kSplitK; ++sp) {
-        if (sp >= nsplit) continue;
-        const float w = ms[sp] == -INFINITY ? 0.f : fast_exp2(ms[sp] - mmax);
-        lsum += w * ls[sp];
+      for (int sp = 0; sp < nsplit; ++sp) {
+        float m_, l_;
+        load_dev(bml + sp * 256 + r * 2, m_, l_);
+        const float w = m_ == -INFINITY ? 0.f : fast_exp2(m_ - mmax);
+        lsum += w * l_;
         const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
         acc[0] += w * x[0]; acc[1] += w * x[1]; acc[2] += w * x[2]; acc[3] += w * x[3];
       }
@@ -312,13 +310,12 @@ void fwd_kernel(const KArgs a) {
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BM = 128, BN = 64;
-  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? split_extra(a.nKs) : 0);
-  const int slots = (a.B * a.H + 7) / 8;
+  const int nQt = (DOC ? a.Pp / BM : (a.M + BM - 1) / BM) + (DOC ? split_extra(a) : 0);
   const size_t lds = 4 * BN * (D < 32 ? 32 : D) * 2 + 2 * BN * 4;  // K, V double buffered + key ids
   auto kern = fwd_kernel<Tag, D, CAUSAL, DOC>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
-  hipLaunchKernelGGL(kern, dim3(8 * slots * nQt), dim3(256), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid_blocks(nQt, a.B * a.H)), dim3(256), lds, s, a);
   return (int)hipGetLastError();
 }
 

@@ -344,10 +344,13 @@ FA_DEV void mask_doc(f32x16& s, const char* ids, int eq_i, bool glob_i, float fi
 
 // ---------------------------------------------------------------------------
 // Work assignment of one workgroup of the forward / dq kernels, including the split of the
-// key range of global-row tiles (kSplitK, fa_common.h).
-//   slots [0, nE)          : chunks 1 .. kSplitK-1 of the first kSplitTiles global-row tiles
+// key range of global-row tiles (SplitCfg, fa_common.h).
+//   slots [0, nE)          : chunks 1 .. split_k-1 of the first split_tiles global-row tiles
 //   slots [nE, nE + nQt)   : every tile, last tile first (chunk 0 when the tile is split)
 // ---------------------------------------------------------------------------
+// Extra workgroup slots per (batch, head): chunks 1 .. split_k-1 of every splittable tile.
+FA_HD int split_extra(const KArgs& a) { return a.split_tiles * (a.split_k - 1); }
+
 struct QWork {
   int tile;    // 128-row tile (natural order, or permuted order with ids)
   int gt;      // index among the splittable global-row tiles, or -1
@@ -359,25 +362,25 @@ FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
   if (!DOC) { w.tile = nQt - 1 - slot; w.gt = -1; w.split = 0; return true; }
   const QHeader hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
   const int g0 = hd.nLp / 128;   // first global-row tile
-  const int nE = split_extra(a.nKs);
+  const int nE = split_extra(a);
   if (slot < nE) {
-    w.gt = slot / (kSplitK - 1);
-    w.split = 1 + slot % (kSplitK - 1);
+    w.gt = slot / (a.split_k - 1);
+    w.split = 1 + slot % (a.split_k - 1);
     w.tile = g0 + w.gt;
     return w.tile < hd.nT128;
   }
   w.tile = nQt - 1 - (slot - nE);
   w.split = 0;
-  w.gt = (w.tile >= g0 && w.tile - g0 < kSplitTiles) ? w.tile - g0 : -1;
+  w.gt = (w.tile >= g0 && w.tile - g0 < a.split_tiles) ? w.tile - g0 : -1;
   return true;
 }
 
 // Cut the key-tile range [first, last) of a splittable tile into chunks; returns the number of
 // chunks in use (1: not split) and narrows [first, last) to this workgroup's chunk.
-FA_DEV int split_range(const QWork& w, int& first, int& last) {
+FA_DEV int split_range(const KArgs& a, const QWork& w, int& first, int& last) {
   if (w.gt < 0) return 1;
   const int n = max(0, last - first);
-  const int ns = min(kSplitK, max(1, n / kSplitMinTiles));
+  const int ns = min(a.split_k, max(1, n / kSplitMinTiles));
   const int c = (n + ns - 1) / ns;
   first = min(last, first + w.split * c);
   last = min(last, first + c);
@@ -428,26 +431,49 @@ FA_DEV bool split_arrive(int* counter, int nsplit) {
   return sk_last != 0;
 }
 
-// blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head).
-// Consecutive workgroup ids land on different XCDs, so every XCD is given whole
-// heads (its L2 then keeps that head's K/V or Q/dO).  Inside an XCD the order is
-//   head-major (tile_major = false): one head after the other -- best L2 reuse when
-//        every tile streams most of the head (no ids);
-//   tile-major (tile_major = true): tile slot 0 of all the XCD's heads, then slot 1, ...
-//        -- with ids the few heavy tiles (global rows) of EVERY head start at once
-//        instead of queueing behind the light tiles of the heads before them.
+// blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head); grid_blocks() is the
+// matching grid size.  Consecutive workgroup ids land on different XCDs (8 of them, each with its
+// own L2), so the map decides which XCD's L2 sees which head:
+//   BH a multiple of 8 : every XCD is given whole heads (its L2 keeps that head's K/V or Q/dO).
+//        Inside an XCD the order is
+//          head-major (tile_major = false): one head after the other -- best L2 reuse when every
+//               tile streams most of the head (no ids);
+//          tile-major (tile_major = true): tile slot 0 of all the XCD's heads, then slot 1, ... --
+//               with ids the few heavy tiles (global rows) of EVERY head start at once instead of
+//               queueing behind the light tiles of the heads before them.
+//   BH = 1, 2, 4      : a head is shared by 8 / BH XCDs, its tile slots dealt round-robin among them
+//                       (heavy and light slots alternate, so the XCDs stay balanced).
+//   otherwise          : (slot, head) pairs dealt round-robin over the XCDs, slot-major: balanced for
+//                       any BH, at the price of every L2 seeing every head.
 // Returns false for padding ids.
+FA_HD int grid_blocks(int ntile, int BH) {
+  if (BH % 8 == 0) return BH * ntile;
+  if (BH < 8 && 8 % BH == 0) { const int k = 8 / BH; return 8 * ((ntile + k - 1) / k); }
+  return (BH * ntile + 7) / 8 * 8;
+}
+
 FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, int& bh) {
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int heads = (BH + 7) / 8;  // heads per XCD
-  if (tile_major) {
-    bh = (idx % heads) * 8 + xcd;
-    tile_slot = idx / heads;
-  } else {
-    bh = (idx / ntile) * 8 + xcd;
-    tile_slot = idx % ntile;
+  if (BH % 8 == 0) {
+    const int heads = BH / 8;  // heads per XCD
+    if (tile_major) {
+      bh = (idx % heads) * 8 + xcd;
+      tile_slot = idx / heads;
+    } else {
+      bh = (idx / ntile) * 8 + xcd;
+      tile_slot = idx % ntile;
+    }
+    return true;
   }
-  return bh < BH;
+  if (BH < 8 && 8 % BH == 0) {
+    const int k = 8 / BH;
+    bh = xcd / k;
+    tile_slot = idx * k + xcd % k;
+    return tile_slot < ntile;
+  }
+  tile_slot = int(blockIdx.x) / BH;
+  bh = int(blockIdx.x) % BH;
+  return tile_slot < ntile;
 }
 
 }  // namespace fa
