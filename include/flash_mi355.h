@@ -124,6 +124,12 @@ int fa_validate(const fa_params* p, int stage);
 /* Bytes of workspace fa_mask_plan needs for these sizes (0 when score_mode == 0). */
 uint64_t fa_workspace_bytes(const fa_params* p);
 
+/* The first fa_workspace_plan_bytes() bytes of the workspace carry the plan from fa_mask_plan to
+   the compute calls (and stay valid after them); the rest is scratch without state between calls.
+   A caller that keeps a plan between forward and backward (as the reference keeps eq/ek,
+   flash_triton.py:557) needs to keep this prefix only and may copy it into a fresh workspace. */
+uint64_t fa_workspace_plan_bytes(const fa_params* p);
+
 /* Mask engine: normalise eq/ek to int32 and build per-tile id summaries
    into p->workspace.  Must be enqueued before fa_fwd / fa_bwd_* on the same
    stream whenever score_mode != 0.  The same workspace serves forward and backward.

@@ -86,6 +86,7 @@ def test_workspace_size():
     want = (r256(128 * 4) + r256(4 * 256 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
             + r256(4 * 4 * 32))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want   # 4 key tiles of 64: no key range is ever split
+    assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want   # ... so all of it is plan
     # from 32 key tiles on, scratch for split global-row tiles: arrival counters, (max, sum) pairs, fp32
     # partial tiles; chunks = clamp(key tiles / 32, 2, 4), splittable tiles = clamp(128 MiB / footprint, 8, 64)
     p.N = 2048
@@ -96,6 +97,9 @@ def test_workspace_size():
             + r256(4 * 32 * 32)
             + r256(4 * tiles * 4) + r256(4 * tiles * chunks * 128 * 2 * 4) + r256(4 * tiles * chunks * 128 * p.D * 4))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want
+    # the plan proper (what has to survive from forward to backward) ends after the counters
+    scratch = r256(4 * tiles * chunks * 128 * 2 * 4) + r256(4 * tiles * chunks * 128 * p.D * 4)
+    assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want - scratch
 
 
 def test_python_layer_asserts_like_the_reference():

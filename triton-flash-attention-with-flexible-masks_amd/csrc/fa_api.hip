@@ -80,6 +80,12 @@ extern "C" uint64_t fa_workspace_bytes(const fa_params* p) {
   return ws_layout(p).total;
 }
 
+extern "C" uint64_t fa_workspace_plan_bytes(const fa_params* p) {
+  if (p == nullptr || p->score_mode == FA_SCORE_MODE0_NOPE) return 0;
+  if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
+  return ws_layout(p).plan_bytes;
+}
+
 static KArgs make_args(const fa_params* p) {
   KArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;

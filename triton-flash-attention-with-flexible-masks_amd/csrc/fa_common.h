@@ -250,6 +250,7 @@ struct WsLayout {
   int nCh;                // row chunks of the partition kernels
   uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum;  // bytes
   uint64_t off_sk_cnt, off_sk_ml, off_sk_o, total;
+  uint64_t plan_bytes;   // leading part that carries state from the plan to the kernels; the rest is scratch
 };
 
 inline WsLayout ws_layout(const fa_params* p) {
@@ -276,6 +277,7 @@ inline WsLayout ws_layout(const fa_params* p) {
   const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
   const uint64_t nsk = uint64_t(p->B) * p->H * sc.tiles;
   w.off_sk_cnt = take(nsk * 4);
+  w.plan_bytes = o;      // the counters (zeroed by the plan, left at zero by every kernel) are state
   w.off_sk_ml = take(nsk * sc.k * 128 * 2 * 4);
   w.off_sk_o = take(nsk * sc.k * 128 * uint64_t(p->D) * 4);
   w.total = o;

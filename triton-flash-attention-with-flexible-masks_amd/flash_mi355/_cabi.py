@@ -22,7 +22,7 @@ FA_IDTYPE_I64 = 1
 # every symbol include/flash_mi355.h declares
 EXPORTS = (
     "fa_version", "fa_params_size", "fa_error_string", "fa_last_hip_error", "fa_validate",
-    "fa_workspace_bytes", "fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq",
+    "fa_workspace_bytes", "fa_workspace_plan_bytes", "fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq",
     "fa_mask_dump",
 )
 
@@ -69,6 +69,8 @@ def lib() -> ctypes.CDLL:
     L.fa_validate.argtypes = [POINTER(FaParams), c_int]
     L.fa_workspace_bytes.restype = c_uint64
     L.fa_workspace_bytes.argtypes = [POINTER(FaParams)]
+    L.fa_workspace_plan_bytes.restype = c_uint64
+    L.fa_workspace_plan_bytes.argtypes = [POINTER(FaParams)]
     for name in ("fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
         fn = getattr(L, name)
         fn.restype = c_int

@@ -79,6 +79,22 @@ class _Plan:
             self.p.workspace_bytes = nbytes
             _cabi.check(L.fa_mask_plan(ctypes.byref(self.p), _stream_ptr(device)), "fa_mask_plan")
 
+    def plan_state(self):
+        """Copy of the part of the workspace that carries the plan (the rest, by far the larger part,
+        is scratch): what the forward keeps for the backward."""
+        if self.workspace is None:
+            return None
+        n = int(_cabi.lib().fa_workspace_plan_bytes(ctypes.byref(self.p)))
+        return self.workspace[:n].clone()
+
+    def restore(self, state, device):
+        """Fresh workspace with a saved plan in front; no planning kernels run."""
+        nbytes = int(_cabi.lib().fa_workspace_bytes(ctypes.byref(self.p)))
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.workspace[:state.numel()].copy_(state)
+        self.p.workspace = self.workspace.data_ptr()
+        self.p.workspace_bytes = nbytes
+
 
 def _prep_ids(e, name):
     assert e.dim() == 3, f"{name} must be [bs, H, L]"
@@ -137,7 +153,7 @@ class FlashAttention(torch.autograd.Function):
             _set4(p.o_stride, Out)
             plan.ensure_workspace(q.device)
             _cabi.check(L.fa_fwd(ctypes.byref(p), _stream_ptr(q.device)), "fa_fwd")
-        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.workspace)
+        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.plan_state())
         ctx.sm_scale = sm_scale
         ctx.causal = causal
         ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
@@ -155,8 +171,7 @@ class FlashAttention(torch.autograd.Function):
             plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode)
             p = plan.p
             if workspace is not None:   # the forward's mask plan is reused as is
-                plan.workspace = workspace
-                p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
+                plan.restore(workspace, q.device)
             delta = torch.empty_like(lse)
             dq = torch.empty_like(q, memory_format=torch.contiguous_format)
             # the dk/dv kernel walks the query heads of a group itself and writes the group sum
