@@ -160,6 +160,29 @@ def test_transposed_views_and_strided_gradients():
         assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
 
 
+def test_lse_output_is_differentiable():
+    """loss = <O, dO> + <LSE, w>: the gradient that arrives at LSE only shifts delta in the backward."""
+    from flash_mi355 import attention_with_lse, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    B, H, L, D = 1, 2, 320, 64
+    g = torch.Generator().manual_seed(31)
+    rng = np.random.default_rng(31)
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g).bfloat16() for _ in range(4))
+    w = torch.randn(B, H, L, generator=g)
+    ek = torch.from_numpy(_ids(rng, B, H, L, "uniform"))[:, None, :].expand(B, H, L)
+    print("case differentiable lse", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out, lse = attention_with_lse(qd, kd, vd, True, None, ek.cuda(), ek.cuda(), SCORE_FUNC_MODE1_DOC)
+    ((out.float() * do.cuda().float()).sum() + (lse * w.cuda()).sum()).backward()
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    ro, rl = O.attention_closed_form(qr, kr, vr, True, None, ek, ek, 1)
+    ((ro * do.float()).sum() + (rl * w).sum()).backward()
+    assert (lse.detach().cpu() - rl.detach()).abs().max().item() <= TOL_LSE
+    for name, got, want in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
+
+
 def test_harness_cell_runs_and_agrees():
     from flash_mi355 import harness as Hn
     torch.manual_seed(5)

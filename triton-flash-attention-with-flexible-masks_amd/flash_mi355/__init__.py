@@ -5,8 +5,8 @@
 
 The four public names match the reference module ``flash_triton``.
 """
-from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, FlashAttention, attention,
+from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, FlashAttention, FlashAttentionWithLse, attention,
                   attention_with_lse, mask_dump, maybe_contiguous)
 
-__all__ = ["attention", "FlashAttention", "SCORE_FUNC_MODE0_NOPE", "SCORE_FUNC_MODE1_DOC",
+__all__ = ["attention", "FlashAttention", "FlashAttentionWithLse", "SCORE_FUNC_MODE0_NOPE", "SCORE_FUNC_MODE1_DOC",
            "attention_with_lse", "mask_dump", "maybe_contiguous"]

@@ -104,8 +104,8 @@ def _prep_ids(e, name):
     return e
 
 
-class FlashAttention(torch.autograd.Function):
-    """Mirror of the reference autograd function (flash_triton.py:506-638)."""
+class _Impl:
+    """Forward and backward shared by the two autograd functions below."""
 
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
@@ -158,10 +158,10 @@ class FlashAttention(torch.autograd.Function):
         ctx.causal = causal
         ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
         ctx.score_func_info = (score_func_mode,)
-        return Out
+        return Out, lse
 
     @staticmethod
-    def backward(ctx, do):
+    def backward(ctx, do, dlse):
         q, k, v, o, lse, eq, ek, workspace = ctx.saved_tensors
         B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
         score_func_mode, = ctx.score_func_info
@@ -184,9 +184,42 @@ class FlashAttention(torch.autograd.Function):
             _set4(p.dq_stride, dq); _set4(p.dk_stride, dk); _set4(p.dv_stride, dv)
             stream = _stream_ptr(q.device)
             _cabi.check(L.fa_bwd_delta(ctypes.byref(p), stream), "fa_bwd_delta")
+            if dlse is not None:
+                # dS = P * (dP - delta) + dLSE * P: a gradient arriving at LSE only shifts delta
+                delta.sub_(torch.where(torch.isinf(lse), torch.zeros_like(lse), dlse.to(torch.float32)))
             _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
             _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
         return dq, dk, dv, None, None, None, None, None
+
+
+_forward, _backward = _Impl.forward, _Impl.backward
+
+
+class FlashAttention(torch.autograd.Function):
+    """Mirror of the reference autograd function (flash_triton.py:506-638)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+        return _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)[0]
+
+    @staticmethod
+    def backward(ctx, do):
+        return _backward(ctx, do, None)
+
+
+class FlashAttentionWithLse(torch.autograd.Function):
+    """Same operator returning (Out, LSE), LSE in natural-log units, both differentiable -- what a
+    caller needs to merge partial attentions over key shards (no counterpart in the reference, whose
+    entry point returns Out only, flash_triton.py:564)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+        out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+        return out, lse * math.log(2.0)
+
+    @staticmethod
+    def backward(ctx, do, dlse):
+        return _backward(ctx, do, dlse)
 
 
 def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE):
@@ -199,14 +232,9 @@ def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func
 # ---------------------------------------------------------------------------
 def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
                        score_func_mode=SCORE_FUNC_MODE0_NOPE):
-    """Forward only; returns (O, LSE) with LSE in natural-log units (-inf for empty rows)."""
-    class _Ctx:
-        def save_for_backward(self, *t):
-            self.saved = t
-    ctx = _Ctx()
-    with torch.no_grad():
-        out = FlashAttention.forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)
-    return out, ctx.saved[4] * math.log(2.0)
+    """(O, LSE) with LSE in natural-log units (-inf for rows without a kept key); differentiable
+    through both results."""
+    return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
 
 
 def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda"):
