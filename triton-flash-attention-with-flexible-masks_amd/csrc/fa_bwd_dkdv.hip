@@ -47,7 +47,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   using Loader = TileLoader<DL, BQ, D, 8>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar
   const int role = wave >> 2, kb = wave & 3;
   const int lq = lane & 31, g = lane >> 5;
 
@@ -122,6 +122,13 @@ void bwd_dkdv_kernel(const KArgs a) {
       if (wave == 0) glb_load_lds4(lsep + r, aux);
       if (wave == 1) glb_load_lds4(delp + r, aux + 256);
     } else {
+      // The row indices were fetched a tile ago and have arrived (the caller waited for every
+      // outstanding load before the barrier).  Tell the compiler so here: the wait it would place
+      // at their first use would otherwise land between / behind the asynchronous loads issued
+      // below and, counting in order, would wait for THOSE as well.
+#pragma unroll
+      for (int i = 0; i < Loader::PER; ++i) settle(ri_t[i]);
+      settle(ri_aux);
 #pragma unroll
       for (int i = 0; i < Loader::PER; ++i) {
         if (Loader::NI % 8 == 0 || i * 8 + wave < Loader::NI) {
