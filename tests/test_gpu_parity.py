@@ -183,6 +183,60 @@ def test_lse_output_is_differentiable():
         assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
 
 
+def test_graph_capture_and_replay():
+    """The five calls of a step (plan, forward, delta, dk/dv, dq) captured into one HIP graph: every
+    replay, with new inputs copied into the captured buffers and eager work in between, must give the
+    eager result bit for bit (the library allocates nothing and clears its counters with kernels)."""
+    import ctypes
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    L = _cabi.lib()
+    B, H, M, D = 1, 4, 2304, 64          # long enough for split key ranges (36 key tiles)
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(41)
+    rng = np.random.default_rng(41)
+    ids = torch.from_numpy(_ids(rng, B, H, M, "uniform")).to(dev)[:, None, :].expand(B, H, M)
+    q, k, v, do = (torch.randn(B, H, M, D, generator=g).bfloat16().to(dev) for _ in range(4))
+    o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    lse = torch.empty(B, H, M, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    plan = _Plan(q, k, v, True, 1.0 / math.sqrt(D), ids, ids, 1)
+    p = plan.p
+    p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+        _set4(getattr(p, f), t)
+    nbytes = int(L.fa_workspace_bytes(ctypes.byref(p)))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+    ref = ctypes.byref(p)
+
+    def step():
+        s = _stream_ptr(dev)
+        for name in ("fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
+            _cabi.check(getattr(L, name)(ref, s), name)
+
+    print("case graph capture", flush=True)
+    step()                       # eager once: kernel attributes are set outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in (q, k, v, do):
+            t.copy_(torch.randn(B, H, M, D, generator=g).bfloat16())
+        step()
+        torch.cuda.synchronize()
+        want = [t.clone() for t in (o, lse, dq, dk, dv)]
+        for t in (o, lse, dq, dk, dv):
+            t.zero_()
+        _ = (q.float() @ k.float().transpose(-1, -2)).sum().item()   # unrelated eager work and a sync in between
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, w_ in zip(("o", "lse", "dq", "dk", "dv"), (o, lse, dq, dk, dv), want):
+            assert torch.equal(got, w_), (rep, name)
+
+
 def test_harness_cell_runs_and_agrees():
     from flash_mi355 import harness as Hn
     torch.manual_seed(5)
