@@ -183,6 +183,15 @@ def test_lse_output_is_differentiable():
         assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
 
 
+def test_negative_and_large_scale():
+    """sm_scale < 0 (the sign moves into Q so that the running maximum stays a maximum) and a large
+    scale (sharp softmax: the lazily moved reference point has to move often)."""
+    _run_case(1, 2, 2, 320, 320, 64, torch.bfloat16, True, True, seed=51, sm_scale=-0.2)
+    _run_case(1, 2, 2, 320, 320, 128, torch.float16, False, False, seed=52, sm_scale=-0.09)
+    _run_case(1, 2, 2, 384, 384, 128, torch.bfloat16, True, True, seed=53, sm_scale=0.25)
+    _run_case(1, 2, 1, 256, 2304, 64, torch.bfloat16, True, True, seed=54, sm_scale=0.3)   # split tiles + sharp softmax
+
+
 def test_graph_capture_and_replay():
     """The five calls of a step (plan, forward, delta, dk/dv, dq) captured into one HIP graph: every
     replay, with new inputs copied into the captured buffers and eager work in between, must give the
