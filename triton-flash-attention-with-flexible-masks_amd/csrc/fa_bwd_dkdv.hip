@@ -1,7 +1,7 @@
 // dK/dV kernel of the split backward.  Replaces _bwd_kv_kernel of the reference
 // (flash_triton.py:175-321).
 //
-// One workgroup = 128 keys, 8 waves.  The two waves that share a SIMD own the SAME 32 keys and
+// One workgroup = 128 keys.  D = 128: 8 waves; the two waves that share a SIMD own the SAME 32 keys and
 // split the work by role, so that each needs only one operand fragment set and one accumulator
 // set (two waves per SIMD fit in the register file, and one role's vector work overlaps the
 // other role's matrix work):
@@ -13,7 +13,7 @@
 // (flash_triton.py:265-308; dK is scaled by sm_scale at the end, :313).  In the accumulator
 // layout each lane owns ONE key column and 16 query rows of every 32-row block, so LSE / delta /
 // eq / row index are read as broadcast 16-byte LDS loads, and P travels between the two roles in
-// exactly the register layout both of them use.
+// exactly the register layout both of them use.  D <= 64: 4 waves, each doing both roles in turn.
 // Query-side tiles (Q, dO, LSE, delta, eq, row index; 64 rows) are streamed through LDS, two
 // buffers.  With document ids the query side is walked in the permuted (local rows first) order
 // of the mask plan: tiles are gathered row by row through the permutation (row indices fetched
@@ -30,8 +30,13 @@
 
 namespace fa {
 
-template <typename Tag, int D, bool CAUSAL, bool DOC>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// SPLIT = true : 8 waves, roles split over the wave pairs as described above (D = 128: one wave cannot
+//                hold both operand sets and both accumulator sets next to a second wave on its SIMD).
+// SPLIT = false: 4 waves, every wave does both roles for its 32 keys (D <= 64: everything fits), so P
+//                never leaves the registers and the only barrier is the one of the tile stream; two
+//                workgroups share a CU.
+template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
@@ -44,11 +49,12 @@ void bwd_dkdv_kernel(const KArgs a) {
   constexpr int AUX_BYTES = 1024;
   constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][4 key blocks][4 x 1024] fp32 P
   constexpr int P_BYTES = 4096;
-  using Loader = TileLoader<DL, BQ, D, 8>;
+  constexpr int NW = SPLIT ? 8 : 4;
+  using Loader = TileLoader<DL, BQ, D, NW>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar
-  const int role = wave >> 2, kb = wave & 3;
+  const int role = SPLIT ? wave >> 2 : 0, kb = wave & 3;
   const int lq = lane & 31, g = lane >> 5;
 
   // one workgroup per (key tile, batch, kv head)
@@ -67,8 +73,16 @@ void bwd_dkdv_kernel(const KArgs a) {
   const T* srcp = role == 0 ? reinterpret_cast<const T*>(a.k) + b * a.k_bs + hk * a.k_hs + int64_t(keyc) * a.k_rs
                             : reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs + int64_t(keyc) * a.v_rs;
   vec8 frag[KS];
+  vec8 frag2[KS];   // V^T next to K^T when one wave does both roles
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) frag[ks] = *reinterpret_cast<const vec8*>(srcp + ks * 16 + g * 8);
+  if (!SPLIT) {
+    const T* vsrc = reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs + int64_t(keyc) * a.v_rs;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) frag2[ks] = *reinterpret_cast<const vec8*>(vsrc + ks * 16 + g * 8);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) settle(frag2[ks]);
+  }
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) settle(frag[ks]);
   const float c = a.scale_log2e;
@@ -92,17 +106,18 @@ void bwd_dkdv_kernel(const KArgs a) {
   int g_coff[Loader::PER], g_rit[Loader::PER];
 #pragma unroll
   for (int i = 0; i < Loader::PER; ++i) {
-    g_rit[i] = ((i * 8 + wave) * Loader::RPI + lane / Loader::CPR) % BQ;
+    g_rit[i] = ((i * NW + wave) * Loader::RPI + lane / Loader::CPR) % BQ;
     const int gc = (lane % Loader::CPR) ^ swz<DL, SWZ_ROW>(g_rit[i]);
     g_coff[i] = gc < D / 8 ? gc * 16 : kOobOffset;
   }
 
   // dV^T (score wave) or dK^T (gradient wave): lane = key column, registers = d rows
-  f32x16 acc[DBN];
+  // (one wave doing both roles: acc = dV^T, acc2 = dK^T)
+  f32x16 acc[DBN], acc2[DBN];
 #pragma unroll
   for (int db = 0; db < DBN; ++db)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+    for (int r = 0; r < 16; ++r) { acc[db][r] = 0.f; acc2[db][r] = 0.f; }
 
   // row indices of a permuted tile this lane needs: PER tile rows for Q/dO, one for the aux arrays
   int ri_t[Loader::PER] = {};
@@ -131,10 +146,10 @@ void bwd_dkdv_kernel(const KArgs a) {
       settle(ri_aux);
 #pragma unroll
       for (int i = 0; i < Loader::PER; ++i) {
-        if (Loader::NI % 8 == 0 || i * 8 + wave < Loader::NI) {
+        if (Loader::NI % NW == 0 || i * NW + wave < Loader::NI) {
           const int r = ri_t[i] >= 0 ? ri_t[i] : 0;
-          buf_load_lds16(ldQ.rsrc, smem + bufi * TILE_BYTES + (i * 8 + wave) * 1024, r * ldQ.row_bytes + g_coff[i], 0);
-          buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * 8 + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
+          buf_load_lds16(ldQ.rsrc, smem + bufi * TILE_BYTES + (i * NW + wave) * 1024, r * ldQ.row_bytes + g_coff[i], 0);
+          buf_load_lds16(ldO.rsrc, smem + (2 + bufi) * TILE_BYTES + (i * NW + wave) * 1024, r * ldO.row_bytes + g_coff[i], 0);
         }
       }
       const int r = ri_aux >= 0 ? ri_aux : 0;
@@ -147,8 +162,51 @@ void bwd_dkdv_kernel(const KArgs a) {
 
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+  // Masks on P of one 32-row block (lane = key column, register 4*q4 + t = row 8*q4 + 4*g + t of the
+  // block); every part sits under a wave-uniform branch.
+  auto mask_p = [&](f32x16& x, const int qb, const int flags, const int tile_id, const int m0, const char* aux)
+                    __attribute__((always_inline)) {
+    const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0, has_glob = (flags & TF_GLOB) != 0;
+    if (need_lim) {
+      // row index inside [first row that may see this key, M); padding rows are -1
+      asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;
+        i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
+        if (DOC) rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          x[4 * q4 + t] = (unsigned)(rowv[t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
+      }
+    }
+    if (DOC && (flags & TF_COL)) {
+      // every row of the tile carries the same local id: the id test depends on the key alone,
+      // i.e. on the lane -- whole columns of the block are kept or dropped
+      asm volatile("" ::: "memory");
+      const bool col_keep = ek_j == tile_id;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[r] = col_keep ? x[r] : 0.f;
+    }
+    if (DOC && need_doc) {
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;
+        const i32x4 eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
+        if (!has_glob) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = eqv[t] == ek_j ? x[4 * q4 + t] : 0.f;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = (eqv[t] >= 0 || eqv[t] == ek_j) ? x[4 * q4 + t] : 0.f;
+        }
+      }
+    }
+  };
+
   // One query tile.  BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
+  auto compute_split = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
     const char* lqt = smem + BUF * TILE_BYTES;
     const char* ldo = smem + (2 + BUF) * TILE_BYTES;
     const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
@@ -158,7 +216,6 @@ void bwd_dkdv_kernel(const KArgs a) {
 
     // wave-level decisions (identical for the two waves of a pair), taken by the tile iterator
     const bool skip = (flags & TF_SKIP) != 0;
-    const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0, has_glob = (flags & TF_GLOB) != 0;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       char* pbuf = smem + P_OFF + (qb * 4 + kb) * P_BYTES + lane * 16;
@@ -191,42 +248,7 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
           }
-          if (need_lim) {
-            // row index inside [first row that may see this key, M); padding rows are -1
-            asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-              const int i0 = 32 * qb + 8 * q4 + 4 * g;
-              i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
-              if (DOC) rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
-#pragma unroll
-              for (int t = 0; t < 4; ++t)
-                x[4 * q4 + t] = (unsigned)(rowv[t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
-            }
-          }
-          if (DOC && (flags & TF_COL)) {
-            // every row of the tile carries the same local id: the id test depends on the key alone,
-            // i.e. on the lane -- whole columns of the block are kept or dropped
-            asm volatile("" ::: "memory");
-            const bool col_keep = ek_j == tile_id;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) x[r] = col_keep ? x[r] : 0.f;
-          }
-          if (DOC && need_doc) {
-            asm volatile("" ::: "memory");
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-              const int i0 = 32 * qb + 8 * q4 + 4 * g;
-              const i32x4 eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
-              if (!has_glob) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) x[4 * q4 + t] = eqv[t] == ek_j ? x[4 * q4 + t] : 0.f;
-              } else {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) x[4 * q4 + t] = (eqv[t] >= 0 || eqv[t] == ek_j) ? x[4 * q4 + t] : 0.f;
-              }
-            }
-          }
+          mask_p(x, qb, flags, tile_id, m0, aux);
           // hand P to the gradient wave of the pair (same lane, same register order)
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4) {
@@ -279,6 +301,90 @@ void bwd_dkdv_kernel(const KArgs a) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+
+  // One query tile, both roles in one wave: S and dP are accumulated alternately, P and dS stay in
+  // registers, then dV^T += dO^T P and dK^T += Q^T dS.
+  auto compute_both = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
+    const char* lqt = smem + BUF * TILE_BYTES;
+    const char* ldo = smem + (2 + BUF) * TILE_BYTES;
+    const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
+    const int m0 = cur * BQ;  // natural order only
+    if (flags & TF_SKIP) return;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      f32x16 x = zero, dp = zero;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 rq = lds_row8<E>(lqt + lo.row[ks] + qb * 32 * DL * 2);
+        x = E::mfma32(rq, frag[ks], x);
+        const vec8 ro = lds_row8<E>(ldo + lo.row[ks] + qb * 32 * DL * 2);
+        dp = E::mfma32(ro, frag2[ks], dp);
+      }
+      {
+        constexpr int NM = 2 * KS, PRE = NM < FA_KV_PRE ? NM : FA_KV_PRE;
+        __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+        for (int i = 0; i < NM - PRE; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // S -> P, masks, dS = P * (dP - delta) for this lane's 16 query rows of the block
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
+        const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
+      }
+      mask_p(x, qb, flags, tile_id, m0, aux);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 32 * qb + 8 * q4 + 4 * g;
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dp[4 * q4 + t] = x[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        vec8 pf, dsf;
+#pragma unroll
+        for (int t = 0; t < 8; t += 2) {
+          const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
+          pf[t] = pr[0]; pf[t + 1] = pr[1];
+          const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
+          dsf[t] = dr[0]; dsf[t + 1] = dr[1];
+        }
+        const int goff = (2 * qb + half) * 16 * DL * 2;
+#pragma unroll
+        for (int db = 0; db < DBN; ++db) {
+          const vec8 to = lds_tr8<E>(ldo + lo.tr[db][0] + goff, ldo + lo.tr[db][1] + goff);
+          acc[db] = E::mfma32(to, pf, acc[db]);
+          const vec8 tq = lds_tr8<E>(lqt + lo.tr[db][0] + goff, lqt + lo.tr[db][1] + goff);
+          acc2[db] = E::mfma32(tq, dsf, acc2[db]);
+        }
+      }
+      {
+        constexpr int NM = 4 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+          if (i % (2 * DBN) == 0) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
+    if constexpr (SPLIT) compute_split(BUF, cur, flags, tile_id);
+    else compute_both(BUF, cur, flags, tile_id);
   };
 
   for (int gi = 0; gi < a.G; ++gi) {
@@ -368,31 +474,39 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
 
   if (key < a.N) {
-    T* orow = role == 0 ? reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs
-                        : reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
-    const float sc = role == 0 ? 1.0f : a.scale;
+    T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs;
+    T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
+    auto store = [&](T* orow, const f32x16 (&v)[DBN], const float sc) __attribute__((always_inline)) {
 #pragma unroll
-    for (int db = 0; db < DBN; ++db)
+      for (int db = 0; db < DBN; ++db)
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
-        const typename E::vec2 k0 = E::cvt2(acc[db][4 * q4 + 0] * sc, acc[db][4 * q4 + 1] * sc);
-        const typename E::vec2 k1 = E::cvt2(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc);
-        typename E::vec4 xk = {k0[0], k0[1], k1[0], k1[1]};
-        *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = xk;
-      }
+        for (int q4 = 0; q4 < 4; ++q4) {
+          if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
+          const typename E::vec2 k0 = E::cvt2(v[db][4 * q4 + 0] * sc, v[db][4 * q4 + 1] * sc);
+          const typename E::vec2 k1 = E::cvt2(v[db][4 * q4 + 2] * sc, v[db][4 * q4 + 3] * sc);
+          typename E::vec4 xk = {k0[0], k0[1], k1[0], k1[1]};
+          *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = xk;
+        }
+    };
+    if (SPLIT) {
+      store(role == 0 ? dvrow : dkrow, acc, role == 0 ? 1.0f : a.scale);
+    } else {
+      store(dvrow, acc, 1.0f);
+      store(dkrow, acc2, a.scale);
+    }
   }
 }
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int BK = 128, BQ = 64;
+  constexpr bool SPLIT = D > 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + 8 * 4096;
-  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC>;
+  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 8 * 4096 : 0);
+  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
-  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(512), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(SPLIT ? 512 : 256), lds, s, a);
   return (int)hipGetLastError();
 }
 
