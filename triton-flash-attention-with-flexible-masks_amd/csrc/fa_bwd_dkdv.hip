@@ -36,7 +36,7 @@ namespace fa {
 //                never leaves the registers and the only barrier is the one of the tile stream; two
 //                workgroups share a CU.
 template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT>
-__global__ __launch_bounds__(SPLIT ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(SPLIT ? 512 : 256) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 3 : 2, D <= 32 ? 3 : 2)))
 void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;

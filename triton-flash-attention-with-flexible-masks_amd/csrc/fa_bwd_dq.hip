@@ -20,7 +20,7 @@
 namespace fa {
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 3 : 2, D <= 64 ? 3 : 2)))
 void bwd_dq_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
