@@ -183,6 +183,30 @@ def test_lse_output_is_differentiable():
         assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
 
 
+@pytest.mark.parametrize("seed", list(range(100, 124)))
+def test_random_shapes(seed):
+    """Seeded draws over the whole argument space of the operator: head size, head counts and groups,
+    ragged and rectangular lengths (down to a single row), causal or not, ids or not, id layouts."""
+    rng = np.random.default_rng(seed)
+    D = int(rng.choice([16, 32, 64, 128]))
+    Hk = int(rng.choice([1, 2, 3]))
+    H = Hk * int(rng.choice([1, 2, 4]))
+    B = int(rng.choice([1, 2]))
+    causal = bool(rng.integers(0, 2))
+    doc = bool(rng.integers(0, 4) > 0)
+    M = int(rng.integers(1, 420))
+    N = int(rng.integers(M, 640)) if (causal or rng.integers(0, 2)) else int(rng.integers(1, 640))
+    if doc and rng.integers(0, 2):
+        N = M   # self-attention with one id vector is the common case
+    if doc and N < M:
+        N = M   # the helper takes the query ids from the tail of the key ids
+    dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float16
+    kind = str(rng.choice(["uniform", "uniform", "alllocal", "allglobal"]))
+    per_head = bool(doc and rng.integers(0, 3) == 0)
+    idt = torch.int64 if rng.integers(0, 2) else torch.int32
+    _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed=seed, ids_kind=kind, per_head_ids=per_head, id_dtype=idt)
+
+
 def test_negative_and_large_scale():
     """sm_scale < 0 (the sign moves into Q so that the running maximum stays a maximum) and a large
     scale (sharp softmax: the lazily moved reference point has to move often)."""
