@@ -1,14 +1,14 @@
 // dK/dV kernel of the split backward.  Replaces _bwd_kv_kernel of the reference
 // (flash_triton.py:175-321).
 //
-// One workgroup = 128 keys.  D = 128: 8 waves; the two waves that share a SIMD own the SAME 32 keys and
-// split the work by role, so that each needs only one operand fragment set and one accumulator
+// One workgroup = 128 keys (64 in the role-split form with document ids, two workgroups per CU).
+// D = 128: two waves per 32 keys; they share a SIMD, own the SAME 32 keys and split the work by role, so that each needs only one operand fragment set and one accumulator
 // set (two waves per SIMD fit in the register file, and one role's vector work overlaps the
 // other role's matrix work):
 //   role 0 ("score" wave)                       role 1 ("gradient" wave)
 //   S  = Q K^T      A = Q rows, B = K^T (regs)  dP = dO V^T     A = dO rows, B = V^T (regs)
 //   P  = exp2(S*c - L), masked -> 0             ---------------- barrier ----------------
-//   P (fp32) -> LDS                             dS = P * (dP - delta)      (P read from LDS)
+//   P (rounded) -> LDS                          dS = P * (dP - delta)      (P read from LDS)
 //   dV^T += dO^T P  A = dO^T (transposed read)  dK^T += Q^T dS  A = Q^T (transposed read)
 // (flash_triton.py:265-308; dK is scaled by sm_scale at the end, :313).  In the accumulator
 // layout each lane owns ONE key column and 16 query rows of every 32-row block, so LSE / delta /
@@ -30,31 +30,33 @@
 
 namespace fa {
 
-// SPLIT = true : 8 waves, roles split over the wave pairs as described above (D = 128: one wave cannot
-//                hold both operand sets and both accumulator sets next to a second wave on its SIMD).
+// SPLIT = true : two waves per block of 32 keys, NKB key blocks per workgroup, roles split over the
+//                wave pairs as described above (D = 128: one wave cannot hold both operand sets and
+//                both accumulator sets next to a second wave on its SIMD).
 // SPLIT = false: 4 waves, every wave does both roles for its 32 keys (D <= 64: everything fits), so P
 //                never leaves the registers and the only barrier is the one of the tile stream; two
 //                workgroups share a CU.
-template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT>
-__global__ __launch_bounds__(SPLIT ? 512 : 256) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 3 : 2, D <= 32 ? 3 : 2)))
+template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT, int NKB>
+__global__ __launch_bounds__(SPLIT ? 128 * NKB : 64 * NKB) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 3 : 2, D <= 32 ? 3 : 2)))
 void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
   using vec8 = typename E::vec8;
-  constexpr int BK = 128, BQ = 64, KS = D / 16;
+  constexpr int BK = 32 * NKB, BQ = 64, KS = D / 16;
   constexpr int DL = D < 32 ? 32 : D;  // LDS row width: D = 16 is staged as 32 columns, the upper 16 zero
   constexpr int DBN = DL / 32;
   constexpr int TILE_BYTES = BQ * DL * 2;
   constexpr int AUX_OFF = 4 * TILE_BYTES;      // [2 buffers][4 arrays][64] x 4 bytes
   constexpr int AUX_BYTES = 1024;
-  constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][4 key blocks][4 x 1024] fp32 P
-  constexpr int P_BYTES = 4096;
-  constexpr int NW = SPLIT ? 8 : 4;
+  constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][NKB key blocks][2 x 1024]: P in the element type
+  constexpr int P_BYTES = 2048;
+  constexpr int NW = SPLIT ? 2 * NKB : NKB;
+  static_assert(NW >= 4, "the four auxiliary arrays of a tile are loaded by waves 0..3");
   using Loader = TileLoader<DL, BQ, D, NW>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar
-  const int role = SPLIT ? wave >> 2 : 0, kb = wave & 3;
+  const int role = SPLIT ? wave / NKB : 0, kb = wave % NKB;
   const int lq = lane & 31, g = lane >> 5;
 
   // one workgroup per (key tile, batch, kv head)
@@ -218,8 +220,9 @@ void bwd_dkdv_kernel(const KArgs a) {
     const bool skip = (flags & TF_SKIP) != 0;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      char* pbuf = smem + P_OFF + (qb * 4 + kb) * P_BYTES + lane * 16;
+      char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
       f32x16 x = zero;
+      vec8 yf[2] = {};   // P (score wave) or dS (gradient wave) of this block, rounded to the element type
       if (!skip) {
         // first product: S (score wave) or dP (gradient wave); operand rows a few LDS reads ahead
         __builtin_amdgcn_sched_barrier(0);
@@ -249,42 +252,48 @@ void bwd_dkdv_kernel(const KArgs a) {
             for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
           }
           mask_p(x, qb, flags, tile_id, m0, aux);
-          // hand P to the gradient wave of the pair (same lane, same register order)
+          // round P for the second product and hand the rounded values to the gradient wave of the
+          // pair (same lane, same register order)
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 pv = {x[4 * q4], x[4 * q4 + 1], x[4 * q4 + 2], x[4 * q4 + 3]};
-            *reinterpret_cast<f32x4*>(pbuf + q4 * 1024) = pv;
+          for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int t = 0; t < 8; t += 2) {
+              const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
+              yf[half][t] = pr[0]; yf[half][t + 1] = pr[1];
+            }
+            *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[half];
           }
         }
       }
       __syncthreads();
       if (!skip) {
         if (role == 1) {
-          // dS = P * (dP - delta)
+          // dS = P * (dP - delta), rounded for the second product
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const int i0 = 32 * qb + 8 * q4 + 4 * g;
-            const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
-            const f32x4 pv = *reinterpret_cast<const f32x4*>(pbuf + q4 * 1024);
+          for (int half = 0; half < 2; ++half) {
+            const f32x8 pv = __builtin_convertvector(*reinterpret_cast<const vec8*>(pbuf + half * 1024), f32x8);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) x[4 * q4 + t] = pv[t] * (x[4 * q4 + t] - dl[t]);
+            for (int q2 = 0; q2 < 2; ++q2) {
+              const int i0 = 32 * qb + 8 * (2 * half + q2) + 4 * g;
+              const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+#pragma unroll
+              for (int t = 0; t < 4; t += 2) {
+                const int e = 4 * q2 + t;
+                const typename E::vec2 pr = E::cvt2(pv[e] * (x[8 * half + e] - dl[t]), pv[e + 1] * (x[8 * half + e + 1] - dl[t + 1]));
+                yf[half][e] = pr[0]; yf[half][e + 1] = pr[1];
+              }
+            }
           }
         }
         // second product: dV^T += dO^T P (score wave) or dK^T += Q^T dS (gradient wave)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-          vec8 yf;
-#pragma unroll
-          for (int t = 0; t < 8; t += 2) {
-            const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
-            yf[t] = pr[0]; yf[t + 1] = pr[1];
-          }
           const int goff = (2 * qb + half) * 16 * DL * 2;
 #pragma unroll
           for (int db = 0; db < DBN; ++db) {
             const vec8 tf = lds_tr8<E>(t2 + lo.tr[db][0] + goff, t2 + lo.tr[db][1] + goff);
-            acc[db] = E::mfma32(tf, yf, acc[db]);
+            acc[db] = E::mfma32(tf, yf[half], acc[db]);
           }
         }
         // transposed fragments (two reads each) a few MFMAs ahead, conversions just in time
@@ -404,7 +413,7 @@ void bwd_dkdv_kernel(const KArgs a) {
       const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
       const IdSummary s0 = ks[n0 / kSumRows];
       gk_lo = s0.lo; gk_hi = s0.hi;
-      if (n0 / kSumRows + 1 < a.nKs) {
+      if (BK > kSumRows && n0 / kSumRows + 1 < a.nKs) {
         const IdSummary s1 = ks[n0 / kSumRows + 1];
         gk_lo = min(gk_lo, s1.lo); gk_hi = max(gk_hi, s1.hi);
       }
@@ -499,14 +508,19 @@ void bwd_dkdv_kernel(const KArgs a) {
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 static int launch_one(const KArgs& a, hipStream_t s) {
-  constexpr int BK = 128, BQ = 64;
   constexpr bool SPLIT = D > 64;
+  // With ids a workgroup visits few query tiles (a dozen at 16K tokens in documents of ~512), so its
+  // set-up and drain are a sizeable part of its life: two 64-key workgroups per CU cover each other's
+  // there (measured 9 % faster); without ids the tile stream is long and the 128-key form reads
+  // every query tile half as often (the 64-key form is 5 % slower there).
+  constexpr int NKB = SPLIT && DOC ? 2 : 4;
+  constexpr int BK = 32 * NKB, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 8 * 4096 : 0);
-  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT>;
+  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 : 0);
+  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT, NKB>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
-  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(SPLIT ? 512 : 256), lds, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(SPLIT ? 128 * NKB : 64 * NKB), lds, s, a);
   return (int)hipGetLastError();
 }
 
