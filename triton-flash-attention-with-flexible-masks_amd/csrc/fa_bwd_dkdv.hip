@@ -27,6 +27,9 @@
 #ifndef FA_KV_PRE2
 #define FA_KV_PRE2 3
 #endif
+#ifndef FA_KV_FLAGSYNC
+#define FA_KV_FLAGSYNC 1
+#endif
 
 namespace fa {
 
@@ -50,6 +53,8 @@ void bwd_dkdv_kernel(const KArgs a) {
   constexpr int AUX_BYTES = 1024;
   constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][NKB key blocks][2 x 1024]: P in the element type
   constexpr int P_BYTES = 2048;
+  constexpr int FLAG_OFF = P_OFF + 2 * NKB * P_BYTES;   // [2 (block parity)][NKB] sequence numbers of the published P
+  constexpr int kPairSpinMax = 1 << 14;   // ~1 ms: orders of magnitude above a legitimate wait
   constexpr int NW = SPLIT ? 2 * NKB : NKB;
   static_assert(NW >= 4, "the four auxiliary arrays of a tile are loaded by waves 0..3");
   using Loader = TileLoader<DL, BQ, D, NW>;
@@ -162,6 +167,8 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
 
+  int pair_seq = 0;   // non-skipped tiles so far: identical in the two waves of a pair
+  if (SPLIT && threadIdx.x < 2 * NKB) *reinterpret_cast<int*>(smem + FLAG_OFF + threadIdx.x * 4) = 0;  // visible after the first tile's barrier
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Masks on P of one 32-row block (lane = key column, register 4*q4 + t = row 8*q4 + 4*g + t of the
@@ -312,6 +319,123 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
 
+  // The same tile with the two roles synchronised pairwise instead of by workgroup barriers: the
+  // score wave publishes P of a 32-row block in LDS and then a sequence number; the gradient wave of
+  // the pair polls that number.  LDS operations of one wave are executed in issue order, so the
+  // number is never visible before P.  Waves of different key blocks drift apart inside a tile
+  // (LDS-heavy and MFMA-heavy phases of different waves overlap); the gradient wave computes dP of
+  // both blocks before it needs the first P.  The wait is bounded, so every wave reaches the end
+  // of the kernel whatever happens.
+  auto compute_flag = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
+    const char* lqt = smem + BUF * TILE_BYTES;
+    const char* ldo = smem + (2 + BUF) * TILE_BYTES;
+    const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
+    const int m0 = cur * BQ;  // natural order only
+    if (flags & TF_SKIP) return;   // decided per wave pair: both roles agree
+    ++pair_seq;
+    auto first_product = [&](const char* rows, const int qb) __attribute__((always_inline)) {
+      f32x16 x = zero;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec8 ra = lds_row8<E>(rows + lo.row[ks] + qb * 32 * DL * 2);
+        x = E::mfma32(ra, frag[ks], x);
+      }
+      {
+        constexpr int PRE = KS < FA_KV_PRE ? KS : FA_KV_PRE;
+        __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+        for (int i = 0; i < KS - PRE; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      return x;
+    };
+    auto second_product = [&](const char* tr, const vec8 (&yf)[2], const int qb) __attribute__((always_inline)) {
+      // NM transposed fragments (two LDS reads each), requested PRE fragments ahead of their MFMA
+      // in program order
+      constexpr int NM = 2 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
+      auto fetch = [&](const int i) __attribute__((always_inline)) {
+        const int half = i / DBN, db = i % DBN;
+        const int goff = (2 * qb + half) * 16 * DL * 2;
+        return lds_tr8<E>(tr + lo.tr[db][0] + goff, tr + lo.tr[db][1] + goff);
+      };
+      __builtin_amdgcn_sched_barrier(0);
+      vec8 tf[NM];
+#pragma unroll
+      for (int i = 0; i < PRE; ++i) tf[i] = fetch(i);
+#pragma unroll
+      for (int i = 0; i < NM; ++i) {
+        if (i + PRE < NM) tf[i + PRE] = fetch(i + PRE);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[i % DBN] = E::mfma32(tf[i], yf[i / DBN], acc[i % DBN]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // Both roles run the same MFMA streams (the accumulators never cross a role branch):
+    //   x0 = first(0) | score: P0 -> LDS | x1 = first(1) | score: P1 -> LDS | gradient: dS0 | second(0) | gradient: dS1 | second(1)
+    // so the gradient wave's first product of block 1 and its second product of block 0 fall into
+    // the score wave's exponentials, and the score wave's second products into the gradient wave's waits.
+    const char* rows = role == 0 ? lqt : ldo;   // rows operand of the first product
+    const char* trp = role == 0 ? ldo : lqt;    // transposed operand of the second product
+    f32x16 x[2];
+    vec8 yf[2][2];   // P (score wave) or dS (gradient wave) per block, rounded to the element type
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      x[qb] = first_product(rows, qb);
+      if (role == 0) {
+        char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
+        // S -> P for this lane's 16 query rows of the block
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
+          const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) x[qb][4 * q4 + t] = fast_exp2(__builtin_fmaf(x[qb][4 * q4 + t], c, -Lv[t]));
+        }
+        mask_p(x[qb], qb, flags, tile_id, m0, aux);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+          for (int t = 0; t < 8; t += 2) {
+            const typename E::vec2 pr = E::cvt2(x[qb][8 * half + t], x[qb][8 * half + t + 1]);
+            yf[qb][half][t] = pr[0]; yf[qb][half][t + 1] = pr[1];
+          }
+          *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[qb][half];
+        }
+        lds_flag_store(smem + FLAG_OFF + (qb * NKB + kb) * 4, pair_seq);
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      if (role == 1) {
+        const char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
+        const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
+        for (int spin = 0; spin < kPairSpinMax && __builtin_amdgcn_readfirstlane(lds_flag_load(fl)) != pair_seq; ++spin) __builtin_amdgcn_s_sleep(1);
+        // dS = P * (dP - delta), rounded for the second product
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const f32x8 pv = __builtin_convertvector(*reinterpret_cast<const vec8*>(pbuf + half * 1024), f32x8);
+#pragma unroll
+          for (int q2 = 0; q2 < 2; ++q2) {
+            const int i0 = 32 * qb + 8 * (2 * half + q2) + 4 * g;
+            const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
+#pragma unroll
+            for (int t = 0; t < 4; t += 2) {
+              const int e = 4 * q2 + t;
+              const typename E::vec2 pr = E::cvt2(pv[e] * (x[qb][8 * half + e] - dl[t]), pv[e + 1] * (x[qb][8 * half + e + 1] - dl[t + 1]));
+              yf[qb][half][e] = pr[0]; yf[qb][half][e + 1] = pr[1];
+            }
+          }
+        }
+      }
+      second_product(trp, yf[qb], qb);
+    }
+  };
+
   // One query tile, both roles in one wave: S and dP are accumulated alternately, P and dS stay in
   // registers, then dV^T += dO^T P and dK^T += Q^T dS.
   auto compute_both = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
@@ -392,7 +516,8 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
   auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
-    if constexpr (SPLIT) compute_split(BUF, cur, flags, tile_id);
+    if constexpr (SPLIT && FA_KV_FLAGSYNC) compute_flag(BUF, cur, flags, tile_id);
+    else if constexpr (SPLIT) compute_split(BUF, cur, flags, tile_id);
     else compute_both(BUF, cur, flags, tile_id);
   };
 
@@ -516,7 +641,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   constexpr int NKB = SPLIT && DOC ? 2 : 4;
   constexpr int BK = 32 * NKB, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 : 0);
+  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 + 64 : 0);
   auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT, NKB>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;

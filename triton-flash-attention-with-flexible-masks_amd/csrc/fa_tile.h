@@ -69,6 +69,20 @@ FA_DEV void glb_load_lds4(const void* src, const char* lds) {
 
 FA_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// A word in LDS used as a flag between two waves of a workgroup.  Explicit LDS instructions: a
+// volatile access through a generic pointer would become a flat access whose completion is
+// counted together with (and so waits for) the asynchronous global -> LDS loads in flight.
+// LDS operations of one wave execute in issue order, so a flag stored after data is never
+// visible before the data.
+FA_DEV void lds_flag_store(const char* p, int v) {
+  asm volatile("ds_write_b32 %0, %1" :: "v"(lds_addr(p)), "v"(v) : "memory");
+}
+FA_DEV int lds_flag_load(const char* p) {
+  int v;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+  return v;
+}
+
 // Global -> LDS tile streamer built on buffer loads with the LDS destination
 // (buffer_load_dwordx4 ... lds).  The per-lane byte offsets are computed once;
 // a tile is then addressed with one scalar offset, and rows past the end of the
