@@ -482,37 +482,42 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) dp[4 * q4 + t] = x[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
       }
-      __builtin_amdgcn_sched_barrier(0);
+      // dV^T += dO^T P and dK^T += Q^T dS alternately: transposed fragments (two LDS reads each) are
+      // requested PRE MFMAs ahead in program order, P and dS are converted just in time; the
+      // scheduling barriers pin that order.
+      {
+        constexpr int NM = 4 * DBN, PRE = NM < FA_KV_PRE2 + 1 ? NM : FA_KV_PRE2 + 1;
+        auto fetch = [&](const int i) __attribute__((always_inline)) {
+          const int half = i / (2 * DBN), db = (i % (2 * DBN)) / 2;
+          const char* t = (i & 1) ? lqt : ldo;
+          const int goff = (2 * qb + half) * 16 * DL * 2;
+          return lds_tr8<E>(t + lo.tr[db][0] + goff, t + lo.tr[db][1] + goff);
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        vec8 tf[NM];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
+        for (int i = 0; i < PRE; ++i) tf[i] = fetch(i);
         vec8 pf, dsf;
 #pragma unroll
-        for (int t = 0; t < 8; t += 2) {
-          const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
-          pf[t] = pr[0]; pf[t + 1] = pr[1];
-          const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
-          dsf[t] = dr[0]; dsf[t + 1] = dr[1];
-        }
-        const int goff = (2 * qb + half) * 16 * DL * 2;
-#pragma unroll
-        for (int db = 0; db < DBN; ++db) {
-          const vec8 to = lds_tr8<E>(ldo + lo.tr[db][0] + goff, ldo + lo.tr[db][1] + goff);
-          acc[db] = E::mfma32(to, pf, acc[db]);
-          const vec8 tq = lds_tr8<E>(lqt + lo.tr[db][0] + goff, lqt + lo.tr[db][1] + goff);
-          acc2[db] = E::mfma32(tq, dsf, acc2[db]);
-        }
-      }
-      {
-        constexpr int NM = 4 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
-#pragma unroll
         for (int i = 0; i < NM; ++i) {
-          if (i % (2 * DBN) == 0) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          if (i + PRE < NM) tf[i + PRE] = fetch(i + PRE);
+          if (i % (2 * DBN) == 0) {
+            const int half = i / (2 * DBN);
+#pragma unroll
+            for (int t = 0; t < 8; t += 2) {
+              const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
+              pf[t] = pr[0]; pf[t + 1] = pr[1];
+              const typename E::vec2 dr = E::cvt2(dp[8 * half + t], dp[8 * half + t + 1]);
+              dsf[t] = dr[0]; dsf[t + 1] = dr[1];
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          const int db = (i % (2 * DBN)) / 2;
+          if (i & 1) acc2[db] = E::mfma32(tf[i], dsf, acc2[db]);
+          else acc[db] = E::mfma32(tf[i], pf, acc[db]);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {

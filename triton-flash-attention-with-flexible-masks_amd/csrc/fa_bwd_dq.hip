@@ -135,35 +135,38 @@ void bwd_dq_kernel(const KArgs a) {
         asm volatile("" ::: "memory");
         mask_doc(s, lid + kb * 32 * 4, eq_i, qc.glob_i, 0.f);
       }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        vec8 dsf;
-#pragma unroll
-        for (int t = 0; t < 8; t += 2) {
-          const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
-          dsf[t] = pr[0];
-          dsf[t + 1] = pr[1];
-        }
-#pragma unroll
-        for (int db = 0; db < DBN; ++db) {
-          const int goff = (2 * kb + half) * 16 * DL * 2;
-          const vec8 ktf = lds_tr8<E>(lk + lo.tr[db][0] + goff, lk + lo.tr[db][1] + goff);
-          dq[db] = E::mfma32(ktf, dsf, dq[db]);
-        }
-      }
-      // K^T fragments (two transposed reads each) a few MFMAs ahead; dS conversions just in time
+      // dQ^T += K^T dS^T: K^T fragments (two transposed reads each) are requested PRE MFMAs ahead in
+      // program order, dS is converted just in time; the scheduling barriers pin that order (left
+      // to itself the scheduler puts every read right before its MFMA).
       {
         constexpr int NM = 2 * DBN, PRE = NM < FA_DQ_PRE2 ? NM : FA_DQ_PRE2;
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
+        auto fetch = [&](const int i) __attribute__((always_inline)) {
+          const int half = i / DBN, db = i % DBN;
+          const int goff = (2 * kb + half) * 16 * DL * 2;
+          return lds_tr8<E>(lk + lo.tr[db][0] + goff, lk + lo.tr[db][1] + goff);
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        vec8 ktf[NM];
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) ktf[i] = fetch(i);
+        vec8 dsf;
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
-          if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          if (i + PRE < NM) ktf[i + PRE] = fetch(i + PRE);
+          if (i % DBN == 0) {
+            const int half = i / DBN;
+#pragma unroll
+            for (int t = 0; t < 8; t += 2) {
+              const typename E::vec2 pr = E::cvt2(s[8 * half + t], s[8 * half + t + 1]);
+              dsf[t] = pr[0];
+              dsf[t + 1] = pr[1];
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          dq[i % DBN] = E::mfma32(ktf[i], dsf, dq[i % DBN]);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
 

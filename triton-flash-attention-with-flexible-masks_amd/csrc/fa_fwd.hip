@@ -22,6 +22,10 @@
 
 #include "fa_tile.h"
 
+#ifndef FA_FWD_PRE2
+#define FA_FWD_PRE2 4
+#endif
+
 namespace fa {
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
@@ -180,32 +184,34 @@ void fwd_kernel(const KArgs a) {
       ps1 += p1;
     }
     l_run += ps0 + ps1;
-    // O^T += V^T P^T, 16 keys per MFMA
-    __builtin_amdgcn_sched_barrier(0);
+    // O^T += V^T P^T, 16 keys per MFMA.  V^T fragments (two transposed reads each) are requested
+    // PRE MFMAs ahead in program order, P is converted just in time; the scheduling barriers pin
+    // that order (left to itself the scheduler puts every read right before its MFMA).
+    {
+      constexpr int NPV = 4 * DBN, PRE = NPV < FA_FWD_PRE2 ? NPV : FA_FWD_PRE2;
+      auto fetch = [&](const int i) __attribute__((always_inline)) {
+        const int c16 = i / DBN, db = i % DBN;
+        return lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * DL * 2, lv + lo.tr[db][1] + c16 * 16 * DL * 2);
+      };
+      __builtin_amdgcn_sched_barrier(0);
+      vec8 vf[NPV];
 #pragma unroll
-    for (int c16 = 0; c16 < 4; ++c16) {
+      for (int i = 0; i < PRE; ++i) vf[i] = fetch(i);
       vec8 pf;
 #pragma unroll
-      for (int t = 0; t < 8; t += 2) {
-        const typename E::vec2 pr = E::cvt2(s[c16 >> 1][8 * (c16 & 1) + t], s[c16 >> 1][8 * (c16 & 1) + t + 1]);
-        pf[t] = pr[0];
-        pf[t + 1] = pr[1];
-      }
-#pragma unroll
-      for (int db = 0; db < DBN; ++db) {
-        const vec8 vf = lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * DL * 2, lv + lo.tr[db][1] + c16 * 16 * DL * 2);
-        o[db] = E::mfma32(vf, pf, o[db]);
-      }
-    }
-    // V^T fragments (two transposed reads each) four MFMAs ahead; P conversions just in time
-    {
-      constexpr int NPV = 4 * DBN, PRE = NPV < 4 ? NPV : 4;
-      __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
-#pragma unroll
       for (int i = 0; i < NPV; ++i) {
-        if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i < NPV - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        if (i + PRE < NPV) vf[i + PRE] = fetch(i + PRE);
+        if (i % DBN == 0) {
+          const int c16 = i / DBN;
+#pragma unroll
+          for (int t = 0; t < 8; t += 2) {
+            const typename E::vec2 pr = E::cvt2(s[c16 >> 1][8 * (c16 & 1) + t], s[c16 >> 1][8 * (c16 & 1) + t + 1]);
+            pf[t] = pr[0];
+            pf[t + 1] = pr[1];
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        o[i % DBN] = E::mfma32(vf[i], pf, o[i % DBN]);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
