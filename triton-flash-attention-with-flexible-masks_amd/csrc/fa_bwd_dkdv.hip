@@ -385,16 +385,21 @@ void bwd_dkdv_kernel(const KArgs a) {
     vec8 yf[2][2];   // P (score wave) or dS (gradient wave) per block, rounded to the element type
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
+      // LSE of this lane's 16 query rows of the block (row 8*q4 + 4*g + t): requested ahead of the
+      // product so that its LDS round trip is hidden
+      f32x4 Lv[4];
+      if (role == 0) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) Lv[q4] = *reinterpret_cast<const f32x4*>(aux + (32 * qb + 8 * q4 + 4 * g) * 4);
+      }
       x[qb] = first_product(rows, qb);
       if (role == 0) {
         char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
-        // S -> P for this lane's 16 query rows of the block
+        // S -> P
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
-          const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
-          const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) x[qb][4 * q4 + t] = fast_exp2(__builtin_fmaf(x[qb][4 * q4 + t], c, -Lv[t]));
+          for (int t = 0; t < 4; ++t) x[qb][4 * q4 + t] = fast_exp2(__builtin_fmaf(x[qb][4 * q4 + t], c, -Lv[q4][t]));
         }
         mask_p(x[qb], qb, flags, tile_id, m0, aux);
 #pragma unroll
@@ -413,20 +418,26 @@ void bwd_dkdv_kernel(const KArgs a) {
     for (int qb = 0; qb < 2; ++qb) {
       if (role == 1) {
         const char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
+        // LDS round trips are long under load: delta is requested before the wait, both halves of
+        // P together after it
+        f32x4 dl[4];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) dl[q4] = *reinterpret_cast<const f32x4*>(aux + 256 + (32 * qb + 8 * q4 + 4 * g) * 4);
         const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
         for (int spin = 0; spin < kPairSpinMax && __builtin_amdgcn_readfirstlane(lds_flag_load(fl)) != pair_seq; ++spin) __builtin_amdgcn_s_sleep(1);
+        vec8 pr8[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const vec8*>(pbuf + half * 1024);
         // dS = P * (dP - delta), rounded for the second product
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-          const f32x8 pv = __builtin_convertvector(*reinterpret_cast<const vec8*>(pbuf + half * 1024), f32x8);
+          const f32x8 pv = __builtin_convertvector(pr8[half], f32x8);
 #pragma unroll
           for (int q2 = 0; q2 < 2; ++q2) {
-            const int i0 = 32 * qb + 8 * (2 * half + q2) + 4 * g;
-            const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
 #pragma unroll
             for (int t = 0; t < 4; t += 2) {
               const int e = 4 * q2 + t;
-              const typename E::vec2 pr = E::cvt2(pv[e] * (x[qb][8 * half + e] - dl[t]), pv[e + 1] * (x[qb][8 * half + e + 1] - dl[t + 1]));
+              const typename E::vec2 pr = E::cvt2(pv[e] * (x[qb][8 * half + e] - dl[2 * half + q2][t]), pv[e + 1] * (x[qb][8 * half + e + 1] - dl[2 * half + q2][t + 1]));
               yf[qb][half][e] = pr[0]; yf[qb][half][e + 1] = pr[1];
             }
           }
