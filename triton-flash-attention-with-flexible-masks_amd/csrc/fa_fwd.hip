@@ -52,9 +52,12 @@ void fwd_kernel(const KArgs a) {
   if (!block_to_tile(nSlots, a.B * a.H, DOC && nQt >= 32, slot, bh)) return;
   const int b = bh / a.H, h = bh % a.H, hk = h / a.G;
   QWork wk;
-  if (!q_work<DOC>(a, b, h, nQt, slot, wk)) return;
+  QHeader hd = {};
+  if (DOC) hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
+  if (!q_work<DOC>(a, hd, nQt, slot, wk)) return;
   QTileCtx<CAUSAL, DOC> qc;
   if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
+  q_work_finish(a, hd, wk);
   int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
   const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
@@ -72,6 +75,14 @@ void fwd_kernel(const KArgs a) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
     qf[ks] = *reinterpret_cast<const vec8*>(qp + int64_t(rowc) * a.q_rs + ks * 16 + g * 8);
+
+  // decisions of this wave for key tile t, evaluated by the lane that tests the tile
+  auto dec = [&](int t, const IdSummary& ks) { return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi), 0); };
+  TileIter it;
+  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);   // its summaries travel together with Q
+
+  // Q has arrived before anything asynchronous is issued (the compiler's in-order wait at its first
+  // use would otherwise also wait for the tile loads issued in between)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) settle(qf[ks]);
   float c = a.scale_log2e;
@@ -80,11 +91,6 @@ void fwd_kernel(const KArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = neg8<E>(qf[ks]);
   }
-
-  // decisions of this wave for key tile t, evaluated by the lane that tests the tile
-  auto dec = [&](int t, const IdSummary& ks) { return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi), 0); };
-  TileIter it;
-  it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);
 
   TileLoader<DL, BN, D> ldK, ldV;
   ldK.init(kp, a.k_rs, a.N);

@@ -371,13 +371,16 @@ struct QWork {
   int split;   // chunk of the key range handled by this workgroup
 };
 
+// The header of the (batch, head) is requested by the caller before this call and, for the common
+// slots [nE, ...), not looked at until q_work_finish: the tile's own summaries and row indices are
+// requested in between, so the two loads overlap instead of forming a dependent chain.
+constexpr int kGtPending = -2;
 template <bool DOC>
-FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
+FA_DEV bool q_work(const KArgs& a, const QHeader& hd, int nQt, int slot, QWork& w) {
   if (!DOC) { w.tile = nQt - 1 - slot; w.gt = -1; w.split = 0; return true; }
-  const QHeader hd = a.qhdr[b * a.qh_bs + h * a.qh_hs];
-  const int g0 = hd.nLp / 128;   // first global-row tile
   const int nE = split_extra(a);
   if (slot < nE) {
+    const int g0 = hd.nLp / 128;   // first global-row tile
     w.gt = slot / (a.split_k - 1);
     w.split = 1 + slot % (a.split_k - 1);
     w.tile = g0 + w.gt;
@@ -385,8 +388,13 @@ FA_DEV bool q_work(const KArgs& a, int b, int h, int nQt, int slot, QWork& w) {
   }
   w.tile = nQt - 1 - (slot - nE);
   w.split = 0;
-  w.gt = (w.tile >= g0 && w.tile - g0 < a.split_tiles) ? w.tile - g0 : -1;
+  w.gt = kGtPending;
   return true;
+}
+FA_DEV void q_work_finish(const KArgs& a, const QHeader& hd, QWork& w) {
+  if (w.gt != kGtPending) return;
+  const int g0 = hd.nLp / 128;
+  w.gt = (w.tile >= g0 && w.tile - g0 < a.split_tiles) ? w.tile - g0 : -1;
 }
 
 // Cut the key-tile range [first, last) of a splittable tile into chunks; returns the number of
