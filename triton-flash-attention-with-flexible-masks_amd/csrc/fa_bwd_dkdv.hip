@@ -177,17 +177,22 @@ void bwd_dkdv_kernel(const KArgs a) {
                     __attribute__((always_inline)) {
     const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0, has_glob = (flags & TF_GLOB) != 0;
     if (need_lim) {
-      // row index inside [first row that may see this key, M); padding rows are -1
+      // row index inside [first row that may see this key, M); padding rows are -1.  The four index
+      // vectors are requested together: one LDS round trip instead of four serial ones.
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
+      i32x4 rowv[4];
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int i0 = 32 * qb + 8 * q4 + 4 * g;
-        i32x4 rowv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
-        if (DOC) rowv = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+        if (DOC) rowv[q4] = *reinterpret_cast<const i32x4*>(aux + 768 + i0 * 4);
+        else rowv[q4] = i32x4{m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};
+      }
+      if (DOC) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-          x[4 * q4 + t] = (unsigned)(rowv[t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
-      }
+          x[4 * q4 + t] = (unsigned)(rowv[q4][t] - row_lo) < row_span ? x[4 * q4 + t] : 0.f;
     }
     if (DOC && (flags & TF_COL)) {
       // every row of the tile carries the same local id: the id test depends on the key alone,
@@ -199,16 +204,18 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
     if (DOC && need_doc) {
       asm volatile("" ::: "memory");
+      i32x4 eqv[4];
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) eqv[q4] = *reinterpret_cast<const i32x4*>(aux + 512 + (32 * qb + 8 * q4 + 4 * g) * 4);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        const int i0 = 32 * qb + 8 * q4 + 4 * g;
-        const i32x4 eqv = *reinterpret_cast<const i32x4*>(aux + 512 + i0 * 4);
         if (!has_glob) {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = eqv[t] == ek_j ? x[4 * q4 + t] : 0.f;
+          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = eqv[q4][t] == ek_j ? x[4 * q4 + t] : 0.f;
         } else {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = (eqv[t] >= 0 || eqv[t] == ek_j) ? x[4 * q4 + t] : 0.f;
+          for (int t = 0; t < 4; ++t) x[4 * q4 + t] = (eqv[q4][t] >= 0 || eqv[q4][t] == ek_j) ? x[4 * q4 + t] : 0.f;
         }
       }
     }

@@ -347,12 +347,17 @@ FA_DEV void mask_lim(f32x16& s, int rel, float fill) {
     for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (8 * q4 + t <= rel) ? s[4 * q4 + t] : fill;
 }
 //   ids  : LDS copy of the block's 32 key ids, already offset by 16*(lane >> 5) bytes
+// The four id vectors are requested together (one LDS round trip instead of four serial ones:
+// left alone, the compiler reuses one register quad and waits after every read).
 FA_DEV void mask_doc(f32x16& s, const char* ids, int eq_i, bool glob_i, float fill) {
+  i32x4 ekv[4];
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) ekv[q4] = *reinterpret_cast<const i32x4*>(ids + 32 * q4);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int q4 = 0; q4 < 4; ++q4) {
-    const i32x4 ekv = *reinterpret_cast<const i32x4*>(ids + 32 * q4);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (glob_i || ekv[t] == eq_i) ? s[4 * q4 + t] : fill;
+    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (glob_i || ekv[q4][t] == eq_i) ? s[4 * q4 + t] : fill;
   }
 }
 
