@@ -375,3 +375,61 @@ def test_device_mask_plan_matches_host_restatement():
                     assert got[7] < got[6]
             for t, s_ in enumerate(P.plan_k(ek[b, h].astype(np.int64), N)):
                 assert (ks[b, h, t, 0], ks[b, h, t, 1]) == (s_["lo"], s_["hi"])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_matches_per_sequence_oracle(causal):
+    """Packed variable-length batch: every sequence against the oracle run on that sequence alone
+    (plain attention, no ids), including an empty sequence, a one-token one and grouped heads."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    lens = [5, 130, 0, 1, 64, 300, 77]
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    T, H, Hk, D = int(cu[-1]), 4, 2, 64
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, Hk, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(T, Hk, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    print(f"varlen lens={lens} causal={causal}", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cu.cuda(), causal=causal)
+    assert out.shape == (T, H, D) and out.is_contiguous()
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for s in range(len(lens)):
+        a, b = int(cu[s]), int(cu[s + 1])
+        if a == b:
+            continue
+        sl = lambda t: t[a:b].transpose(0, 1)[None]          # [1, heads, len, D]
+        ro, _, rdq, rdk, rdv = O.attention_autograd(sl(q), sl(k), sl(v), sl(do), causal, None, None, None, 0)
+        for name, got, ref in (("o", out.detach(), ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+            err = (sl(got.float().cpu()) - ref).abs().max().item()
+            assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), f"sequence {s} {name} err {err}"
+
+
+def test_varlen_cross_attention_and_refusal():
+    """Different query and key boundaries (non-causal): each query sequence sees the keys of the
+    sequence with the same number; the causal form of that case is refused."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    lq, lk = [40, 3, 100], [17, 200, 64]
+    cuq = torch.tensor(np.concatenate([[0], np.cumsum(lq)]), dtype=torch.int32)
+    cuk = torch.tensor(np.concatenate([[0], np.cumsum(lk)]), dtype=torch.int32)
+    Tq, Tk, H, D = int(cuq[-1]), int(cuk[-1]), 2, 128
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(Tq, H, D, generator=g).to(torch.float16)
+    k = torch.randn(Tk, H, D, generator=g).to(torch.float16)
+    v = torch.randn(Tk, H, D, generator=g).to(torch.float16)
+    print("varlen cross", flush=True)
+    out = attention_varlen(q.cuda(), k.cuda(), v.cuda(), cuq.cuda(), cuk.cuda())
+    torch.cuda.synchronize()
+    for s in range(3):
+        qs = q[int(cuq[s]):int(cuq[s + 1])].transpose(0, 1)[None]
+        ks = k[int(cuk[s]):int(cuk[s + 1])].transpose(0, 1)[None]
+        vs = v[int(cuk[s]):int(cuk[s + 1])].transpose(0, 1)[None]
+        ro, _ = O.attention_closed_form(qs, ks, vs, False, None, None, None, 0)
+        got = out[int(cuq[s]):int(cuq[s + 1])].transpose(0, 1)[None].float().cpu()
+        assert (got - ro).abs().max().item() <= TOL_O
+    with pytest.raises(NotImplementedError):
+        attention_varlen(q.cuda(), k.cuda(), v.cuda(), cuq.cuda(), cuk.cuda(), causal=True)

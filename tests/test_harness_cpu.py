@@ -51,3 +51,18 @@ def test_pivot_layout():
     lines = txt.splitlines()
     assert "L=04,D=bf16" in lines[0] and "L=16,D=bf16" in lines[0]
     assert lines[1].startswith("Mode=fwd,C=True,F=a") and "1.50" in lines[1] and "2.50" in lines[1]
+
+
+def test_varlen_ids_mark_sequences():
+    """Packed-batch ids: one negative id per sequence, empty sequences skipped, tokens behind the
+    last boundary in a sequence of their own; two tokens see each other iff their ids are equal,
+    which is the block-diagonal mask of the packed batch (brute force)."""
+    import torch
+    from flash_mi355 import varlen_ids
+    cu = torch.tensor([0, 3, 3, 7, 8], dtype=torch.int32)
+    ids = varlen_ids(cu, 10)
+    assert ids.dtype == torch.int32 and (ids < 0).all()
+    want = [0, 0, 0, 2, 2, 2, 2, 3, 4, 4]          # sequence number of every token
+    for i in range(10):
+        for j in range(10):
+            assert bool(ids[i] == ids[j]) == (want[i] == want[j])

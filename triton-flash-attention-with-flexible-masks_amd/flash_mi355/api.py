@@ -146,7 +146,7 @@ class _Impl:
         L = _cabi.lib()
         with torch.cuda.device(q.device):
             plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
-            Out = torch.empty_like(q, memory_format=torch.contiguous_format)
+            Out = torch.empty_like(q)   # q's layout when q is dense (flash_triton.py:539), contiguous otherwise
             lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
             p = plan.p
             p.o, p.lse = Out.data_ptr(), lse.data_ptr()
@@ -173,7 +173,7 @@ class _Impl:
             if workspace is not None:   # the forward's mask plan is reused as is
                 plan.restore(workspace, q.device)
             delta = torch.empty_like(lse)
-            dq = torch.empty_like(q, memory_format=torch.contiguous_format)
+            dq = torch.empty_like(q)
             # the dk/dv kernel walks the query heads of a group itself and writes the group sum
             # (the reference writes per query head and sums afterwards, flash_triton.py:594-595,635-637)
             dk = torch.empty((B, Hk, N, D), dtype=k.dtype, device=q.device)
@@ -235,6 +235,43 @@ def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
     """(O, LSE) with LSE in natural-log units (-inf for rows without a kept key); differentiable
     through both results."""
     return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+
+
+def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
+    """Document ids of a packed batch: token t of sequence s (cu_seqlens[s] <= t < cu_seqlens[s+1])
+    gets the local id -(s+1); tokens behind the last boundary get the id of a further sequence of
+    their own.  int32, shape [total]."""
+    pos = torch.arange(total, device=cu_seqlens.device, dtype=cu_seqlens.dtype)
+    seq = torch.bucketize(pos, cu_seqlens[1:].contiguous(), right=True)
+    return (-(seq + 1)).to(torch.int32)
+
+
+def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_scale=None):
+    """Packed variable-length batch (the calling convention of varlen flash-attention kernels):
+    q [total_q, H, D], k and v [total_k, Hk, D], cu_seqlens_* int tensors [S+1] of cumulative
+    sequence lengths starting at 0.  Token i of sequence s attends to the keys of sequence s
+    only.  Returns [total_q, H, D]; differentiable.
+
+    The packed batch IS the document mask of the operator: one (batch) row of total_* tokens whose
+    ids are the negated sequence numbers, so no padding and no copy -- q, k, v are passed as
+    [1, H, total, D] views.  causal=True needs cu_seqlens_k to be cu_seqlens_q (self-attention,
+    where the causal bound of the packed row and of every sequence coincide); with different
+    boundaries the per-sequence bottom-right alignment is not a single offset and is refused.
+    (No counterpart in the reference, which takes eq/ek directly, flash_triton.py:506.)"""
+    assert q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be [total, heads, D]"
+    same = cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q
+    if not same and causal:
+        same = cu_seqlens_k.shape == cu_seqlens_q.shape and bool(torch.equal(cu_seqlens_k, cu_seqlens_q))
+        if not same:
+            raise NotImplementedError("causal attention over packed sequences needs cu_seqlens_k == cu_seqlens_q")
+    Tq, H, _ = q.shape
+    Tk = k.shape[0]
+    eq = varlen_ids(cu_seqlens_q, Tq)
+    ek = eq if (same and Tk == Tq) else varlen_ids(cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k, Tk)
+    q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (q, k, v))
+    out = attention(q4, k4, v4, causal, sm_scale, eq.view(1, 1, Tq).expand(1, H, Tq), ek.view(1, 1, Tk).expand(1, H, Tk),
+                    SCORE_FUNC_MODE1_DOC)
+    return out.squeeze(0).transpose(0, 1)
 
 
 def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda"):
