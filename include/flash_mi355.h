@@ -33,7 +33,8 @@
  *                                       including 0
  * Strides are in elements.  The innermost stride of every 4-D tensor must be 1
  * (the reference forces that with maybe_contiguous, flash_triton.py:435-437,525).
- * Base pointers must be 16-byte aligned and row strides multiples of 8 elements.
+ * Base pointers must be 16-byte aligned and outer strides multiples of 16 bytes
+ * (8 elements of a 16-bit type, 4 of fp32).
  */
 #ifndef FLASH_MI355_H
 #define FLASH_MI355_H
@@ -54,6 +55,7 @@ extern "C" {
 /* element types */
 #define FA_DTYPE_BF16 0
 #define FA_DTYPE_FP16 1
+#define FA_DTYPE_FP32 2   /* fp32 tensors: fp32 MFMA throughout (the reference takes fp32 like any float type) */
 #define FA_IDTYPE_I32 0
 #define FA_IDTYPE_I64 1
 

@@ -28,7 +28,7 @@ def _ids(rng, B, H, L, kind):
 
 
 def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
-              id_dtype=torch.int32, sm_scale=None, check_bwd=True):
+              id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE):
     from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
     from oracle import attention_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -64,8 +64,8 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
     lse_err = (lse.cpu()[~dead] - ref_lse[~dead]).abs().max().item() if (~dead).any() else 0.0
     o_err = (out.float().cpu() - ref_o).abs().max().item()
     assert not torch.isnan(out).any()
-    assert lse_err <= TOL_LSE, f"LSE err {lse_err}"
-    assert o_err <= TOL_O, f"O err {o_err}"
+    assert lse_err <= tol_lse, f"LSE err {lse_err}"
+    assert o_err <= tol_o, f"O err {o_err}"
     if not check_bwd:
         return
     out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode)
@@ -79,7 +79,7 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
         # the gradient itself is rounded to bf16/fp16 on output: half an ulp at magnitude x
         # is x * 2^-9, so the absolute bound grows with the gradient's magnitude above 4
         scale = max(1.0, ref.abs().max().item() / 4)
-        assert err <= TOL_O * scale, f"{name} err {err} (ref max {ref.abs().max().item()})"
+        assert err <= tol_o * scale, f"{name} err {err} (ref max {ref.abs().max().item()})"
 
 
 CASES = [
@@ -433,3 +433,30 @@ def test_varlen_cross_attention_and_refusal():
         assert (got - ro).abs().max().item() <= TOL_O
     with pytest.raises(NotImplementedError):
         attention_varlen(q.cuda(), k.cuda(), v.cuda(), cuq.cuda(), cuk.cuda(), causal=True)
+
+
+# fp32 tensors run on fp32 MFMAs: the oracle is fp32 too, so the bound is a few ulps of the
+# accumulated sums, not the 16-bit rounding of the other cases
+TOL_F32 = 2e-4
+FP32_CASES = [
+    # B, H, Hk, M, N, D, causal, doc
+    (2, 4, 4, 512, 512, 64, True, True),       # the reference's own CPU-runnable configuration
+    (1, 2, 2, 256, 256, 128, True, False),
+    (1, 2, 2, 200, 200, 128, False, True),     # ragged
+    (1, 4, 2, 130, 130, 128, True, True),      # grouped-query, ragged
+    (1, 2, 2, 77, 333, 64, True, True),        # rectangular, bottom-right causal
+    (1, 2, 2, 96, 96, 32, True, True),
+    (2, 2, 1, 100, 300, 16, True, True),
+    (1, 1, 1, 1, 1, 16, False, False),
+]
+
+
+@pytest.mark.parametrize("case", FP32_CASES, ids=lambda c: "f32-B%d-H%d-%d-M%d-N%d-D%d-c%d-d%d" % tuple(int(x) for x in c))
+def test_fp32_tensors(case):
+    B, H, Hk, M, N, D, causal, doc = case
+    _run_case(B, H, Hk, M, N, D, torch.float32, causal, doc, seed=5, tol_o=TOL_F32, tol_lse=TOL_F32)
+
+
+def test_fp32_all_global_and_all_local_ids():
+    _run_case(1, 2, 2, 160, 160, 64, torch.float32, True, True, seed=6, ids_kind="allglobal", tol_o=TOL_F32, tol_lse=TOL_F32)
+    _run_case(1, 2, 2, 160, 160, 64, torch.float32, False, True, seed=6, ids_kind="alllocal", tol_o=TOL_F32, tol_lse=TOL_F32)

@@ -11,12 +11,13 @@ static bool d_supported(int D) { return D == 16 || D == 32 || D == 64 || D == 12
 
 // rows/D: extent of one (batch, head) slice; the kernels address a slice through a
 // buffer resource whose byte range must stay below 2 GiB
-static int check_tensor(const void* ptr, const int64_t* st, int rows, int D) {
+static int check_tensor(const void* ptr, const int64_t* st, int rows, int D, int dtype) {
+  const int esize = dtype == FA_DTYPE_FP32 ? 4 : 2, per16 = 16 / esize;
   if (ptr == nullptr) return FA_ERR_NULLPTR;
-  if (st[2] < 0 || (int64_t(rows - 1) * st[2] + D) * 2 >= (int64_t(1) << 31)) return FA_ERR_NOT_IMPLEMENTED;
+  if (st[2] < 0 || (int64_t(rows - 1) * st[2] + D) * esize >= (int64_t(1) << 31)) return FA_ERR_NOT_IMPLEMENTED;
   if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0) return FA_ERR_ALIGN;
   if (st[3] != 1) return FA_ERR_STRIDE;
-  if ((st[0] % 8) != 0 || (st[1] % 8) != 0 || (st[2] % 8) != 0) return FA_ERR_ALIGN;
+  if ((st[0] % per16) != 0 || (st[1] % per16) != 0 || (st[2] % per16) != 0) return FA_ERR_ALIGN;
   return FA_OK;
 }
 
@@ -31,7 +32,7 @@ extern "C" const char* fa_error_string(int code) {
     case FA_ERR_UNSUPPORTED_D: return "head dimension must be one of 16, 32, 64, 128";
     case FA_ERR_DTYPE: return "unsupported element or id type";
     case FA_ERR_SHAPE: return "inconsistent sizes (H % Hk != 0, causal with N < M, or a size <= 0)";
-    case FA_ERR_ALIGN: return "pointers must be 16-byte aligned and outer strides multiples of 8 elements";
+    case FA_ERR_ALIGN: return "pointers must be 16-byte aligned and outer strides multiples of 16 bytes";
     case FA_ERR_STRIDE: return "innermost stride must be 1";
     case FA_ERR_MODE: return "unknown score mode, or doc mode without eq/ek";
     case FA_ERR_WORKSPACE: return "workspace missing or too small";
@@ -44,7 +45,7 @@ extern "C" const char* fa_error_string(int code) {
 extern "C" int fa_validate(const fa_params* p, int stage) {
   if (p == nullptr) return FA_ERR_NULLPTR;
   if (!d_supported(p->D)) return FA_ERR_UNSUPPORTED_D;
-  if (p->dtype != FA_DTYPE_BF16 && p->dtype != FA_DTYPE_FP16) return FA_ERR_DTYPE;
+  if (p->dtype != FA_DTYPE_BF16 && p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_FP32) return FA_ERR_DTYPE;
   if (p->B <= 0 || p->H <= 0 || p->Hk <= 0 || p->M <= 0 || p->N <= 0) return FA_ERR_SHAPE;
   if (p->H % p->Hk != 0) return FA_ERR_SHAPE;
   if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
@@ -59,16 +60,16 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   }
   if (stage == 2) return FA_OK;
   int rc;
-  if ((rc = check_tensor(p->q, p->q_stride, p->M, p->D)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->k, p->k_stride, p->N, p->D)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->v, p->v_stride, p->N, p->D)) != FA_OK) return rc;
-  if ((rc = check_tensor(p->o, p->o_stride, p->M, p->D)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->q, p->q_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->k, p->k_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->v, p->v_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
+  if ((rc = check_tensor(p->o, p->o_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
   if (p->lse == nullptr) return FA_ERR_NULLPTR;
   if (stage == 1) {
-    if ((rc = check_tensor(p->dout, p->do_stride, p->M, p->D)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dq, p->dq_stride, p->M, p->D)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dk, p->dk_stride, p->N, p->D)) != FA_OK) return rc;
-    if ((rc = check_tensor(p->dv, p->dv_stride, p->N, p->D)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dout, p->do_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dq, p->dq_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dk, p->dk_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
+    if ((rc = check_tensor(p->dv, p->dv_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
     if (p->delta == nullptr) return FA_ERR_NULLPTR;
   }
   return FA_OK;
@@ -151,28 +152,36 @@ extern "C" int fa_mask_plan(const fa_params* p, void* stream) {
 extern "C" int fa_fwd(const fa_params* p, void* stream) {
   int rc = fa_validate(p, 0);
   if (rc != FA_OK) return rc;
-  return finish(launch_fwd(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
-                           reinterpret_cast<hipStream_t>(stream)));
+  const bool causal = p->causal != 0, doc = p->score_mode == FA_SCORE_MODE1_DOC;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (p->dtype == FA_DTYPE_FP32) return finish(launch_fwd_f32(make_args(p), p->D, causal, doc, s));
+  return finish(launch_fwd(make_args(p), p->dtype, p->D, causal, doc, s));
 }
 
 extern "C" int fa_bwd_delta(const fa_params* p, void* stream) {
   int rc = fa_validate(p, 1);
   if (rc != FA_OK) return rc;
-  return finish(launch_bwd_delta(make_args(p), p->dtype, p->D, reinterpret_cast<hipStream_t>(stream)));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (p->dtype == FA_DTYPE_FP32) return finish(launch_bwd_delta_f32(make_args(p), p->D, s));
+  return finish(launch_bwd_delta(make_args(p), p->dtype, p->D, s));
 }
 
 extern "C" int fa_bwd_dkdv(const fa_params* p, void* stream) {
   int rc = fa_validate(p, 1);
   if (rc != FA_OK) return rc;
-  return finish(launch_bwd_dkdv(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
-                                reinterpret_cast<hipStream_t>(stream)));
+  const bool causal = p->causal != 0, doc = p->score_mode == FA_SCORE_MODE1_DOC;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (p->dtype == FA_DTYPE_FP32) return finish(launch_bwd_dkdv_f32(make_args(p), p->D, causal, doc, s));
+  return finish(launch_bwd_dkdv(make_args(p), p->dtype, p->D, causal, doc, s));
 }
 
 extern "C" int fa_bwd_dq(const fa_params* p, void* stream) {
   int rc = fa_validate(p, 1);
   if (rc != FA_OK) return rc;
-  return finish(launch_bwd_dq(make_args(p), p->dtype, p->D, p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC,
-                              reinterpret_cast<hipStream_t>(stream)));
+  const bool causal = p->causal != 0, doc = p->score_mode == FA_SCORE_MODE1_DOC;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (p->dtype == FA_DTYPE_FP32) return finish(launch_bwd_dq_f32(make_args(p), p->D, causal, doc, s));
+  return finish(launch_bwd_dq(make_args(p), p->dtype, p->D, causal, doc, s));
 }
 
 extern "C" int fa_mask_dump(const fa_params* p, uint8_t* out, void* stream) {

@@ -305,6 +305,11 @@ int launch_fwd(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStrea
 int launch_bwd_delta(const KArgs& a, int dtype, int D, hipStream_t s);
 int launch_bwd_dq(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
 int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+// the same four for fp32 tensors (fa_f32.hip)
+int launch_fwd_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s);
+int launch_bwd_delta_f32(const KArgs& a, int D, hipStream_t s);
+int launch_bwd_dq_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s);
+int launch_bwd_dkdv_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s);
 int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s);
 int launch_mask_dump(const KArgs& a, bool causal, bool doc, uint8_t* out, hipStream_t s);
 

@@ -1,0 +1,545 @@
+// The operator for fp32 tensors: forward, delta, dk/dv and dq with `v_mfma_f32_32x32x2_f32`
+// (products and accumulation in fp32 throughout).  The reference accepts fp32 tensors like any
+// other float type (flash_triton.py:508-564 has no dtype check; its score and probability
+// matrices then stay fp32, :88,126) -- this is that case, at full fp32 precision.
+//
+// Shape of all three kernels: 4 waves per workgroup, ONE wave per SIMD, so that a wave may use the
+// whole 512-entry register file: the operands of the side a wave owns (32 query rows, or 32 keys)
+// and its accumulators stay in registers for the whole kernel; the other side is streamed through
+// LDS in tiles of 32 rows (the next tile travels global -> registers while the current one is
+// used).  A 32x32x2 MFMA takes ONE operand element per lane, so every operand read from LDS is a
+// single `ds_read_b32` per lane and a transposed operand costs the same as a plain one: rows are
+// padded to D + 1 floats, which makes both access patterns conflict-free.
+//   forward  S^T = K Q^T | online softmax (exp2 domain) | O^T += V^T P^T          flash_triton.py:26-172
+//   dq       S^T = K Q^T, dP^T = V dO^T | dS = P (dP - delta) | dQ^T += K^T dS^T  flash_triton.py:325-433
+//   dk/dv    S = Q K^T, dP = dO V^T | P, dS | dV^T += dO^T P, dK^T += Q^T dS      flash_triton.py:175-321
+// In the accumulator layout of a 32x32 MFMA a lane owns one column (its query row, or its key) and
+// rows 8*q4 + 4*(lane/32) + t; P^T / dS^T / P / dS are consumed as the B operand of the next
+// product straight from those registers (the contraction index is walked in that same order on
+// the A side), so nothing is exchanged or transposed.
+// Masks: rows are walked in natural order; the element masks are the routines of the 16-bit
+// kernels (same accumulator layout); a wave skips a 32x32 block when the causal bound or the id
+// intervals of its rows and of the block's keys (reduced from the ids staged with the tile)
+// exclude every pair.  With ids the int32 id copies of the mask plan are used (fa_mask_plan
+// must have run, as for the other types).
+#include "fa_tile.h"
+
+namespace fa {
+namespace {
+
+FA_DEV f32x16 mfma_f32(float a, float b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+
+constexpr int kRows = 32;       // rows of a streamed tile
+constexpr int kThreads = 256;
+
+// A [32 x D] tile on its way from global memory to LDS, held in registers in between.
+template <int D>
+struct TileRegs {
+  static constexpr int C4 = D / 4, N4 = kRows * C4, PER = (N4 + kThreads - 1) / kThreads;
+  f32x4 v[PER];
+  // rows row0 .. row0+31 of a matrix with `nrows` rows; rows past the end read as zero
+  FA_DEV void load(const float* base, int64_t rs, int row0, int nrows) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + kThreads * i;
+      const int r = idx / C4, c4 = idx % C4;
+      const bool ok = idx < N4 && row0 + r < nrows;
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      v[i] = ok ? *reinterpret_cast<const f32x4*>(base + int64_t(row0 + r) * rs + 4 * c4) : z;
+    }
+  }
+  FA_DEV void store(float* lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + kThreads * i;
+      const int r = idx / C4, c4 = idx % C4;
+      if (idx < N4) {
+        float* d = lds + r * (D + 1) + 4 * c4;
+        d[0] = v[i][0]; d[1] = v[i][1]; d[2] = v[i][2]; d[3] = v[i][3];
+      }
+    }
+  }
+};
+
+// min / max over the 32 lanes of a half wave (both halves hold the same 32 rows)
+FA_DEV int half_min(int x) {
+#pragma unroll
+  for (int off = 16; off >= 1; off >>= 1) x = min(x, __shfl_xor(x, off));
+  return x;
+}
+FA_DEV int half_max(int x) {
+#pragma unroll
+  for (int off = 16; off >= 1; off >>= 1) x = max(x, __shfl_xor(x, off));
+  return x;
+}
+
+template <int D>
+constexpr size_t lds_bytes() { return size_t(2 * kRows * (D + 1) + 4 * kRows + 64) * 4; }
+
+// ---------------------------------------------------------------------------------------------
+template <int D, bool CAUSAL, bool DOC>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void fwd_f32_kernel(const KArgs a) {
+  constexpr int RS = D + 1, KS2 = D / 2, DBN = (D + 31) / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* lk = reinterpret_cast<float*>(smem);
+  float* lv = lk + kRows * RS;
+  int* lid = reinterpret_cast<int*>(lv + kRows * RS);
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lq = lane & 31, g = lane >> 5;
+  const int BH = a.B * a.H;
+  const int nQt = (a.M + 127) / 128;
+  const int tile = nQt - 1 - blockIdx.x / BH;   // the last rows see the most keys: first
+  const int bh = blockIdx.x % BH, b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  const int m0 = tile * 128, mw = m0 + wave * 32;
+  const int row = mw + lq, rowc = min(row, a.M - 1);
+
+  const float* qp = reinterpret_cast<const float*>(a.q) + b * a.q_bs + h * a.q_hs + int64_t(rowc) * a.q_rs;
+  const float* kp = reinterpret_cast<const float*>(a.k) + b * a.k_bs + hk * a.k_hs;
+  const float* vp = reinterpret_cast<const float*>(a.v) + b * a.v_bs + hk * a.v_hs;
+  const int* ekp = DOC ? a.ek32 + b * a.ek_bs + h * a.ek_hs : nullptr;
+
+  float c = a.scale_log2e;
+  float qreg[KS2];   // B operand of S^T = K Q^T: Q[row][2*s + g]
+#pragma unroll
+  for (int s = 0; s < KS2; ++s) qreg[s] = qp[2 * s + g];
+  if (c < 0.f) {     // keep max(raw score) == max(scaled score): move the sign into Q
+    c = -c;
+#pragma unroll
+    for (int s = 0; s < KS2; ++s) qreg[s] = -qreg[s];
+  }
+  const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
+  const bool glob_i = eq_i >= 0;
+  const int lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;   // last key this row may see
+  // the wave's rows: largest such limit, id interval of the local rows, any global row
+  const int w_last = min(mw + 31, a.M - 1);
+  const int w_lim = CAUSAL ? min(a.gap + w_last, a.N - 1) : a.N - 1;
+  int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
+  if (DOC) {
+    const bool live = row < a.M;
+    w_lo = half_min(live && !glob_i ? eq_i : 0x7fffffff);
+    w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
+    w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
+  }
+  const int n_end = CAUSAL ? min(a.N, a.gap + min(m0 + 127, a.M - 1) + 1) : a.N;
+  const int nkt = (n_end + kRows - 1) / kRows;   // the same for all waves: the tile stream has barriers
+
+  f32x16 o[DBN];
+#pragma unroll
+  for (int db = 0; db < DBN; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;   // running reference point (scaled) and this lane's partial row sum
+
+  TileRegs<D> rk, rv;
+  int rid = 0;
+  rk.load(kp, a.k_rs, 0, a.N);
+  rv.load(vp, a.v_rs, 0, a.N);
+  if (DOC && threadIdx.x < kRows) rid = ekp[min((int)threadIdx.x, a.N - 1)];
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int n0 = kt * kRows;
+    __syncthreads();   // the previous tile is no longer read
+    rk.store(lk);
+    rv.store(lv);
+    if (DOC && threadIdx.x < kRows) lid[threadIdx.x] = rid;
+    __syncthreads();
+    if (kt + 1 < nkt) {   // the next tile travels while this one is used
+      rk.load(kp, a.k_rs, n0 + kRows, a.N);
+      rv.load(vp, a.v_rs, n0 + kRows, a.N);
+      if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
+    }
+    bool skip = mw >= a.M || n0 > w_lim;
+    if (DOC && !skip) {
+      const bool kv = n0 + lq < a.N;
+      const int id = lid[lq];
+      const int k_lo = half_min(kv ? id : 0x7fffffff), k_hi = half_max(kv ? id : (int)0x80000000);
+      skip = !doc_may_keep(w_lo, w_hi, w_glob, k_lo, k_hi);
+    }
+    if (skip) continue;
+
+    f32x16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+    for (int st = 0; st < KS2; ++st) s = mfma_f32(lk[lq * RS + 2 * st + g], qreg[st], s);
+    mask_lim(s, lim_i - n0 - 4 * g, -INFINITY);
+    if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, -INFINITY);
+
+    float mx = s[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
+    mx = xhalf_max(mx) * c;                 // -inf stays -inf (c > 0)
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
+    const float msub = (m_new == -INFINITY) ? 0.f : m_new;   // nothing kept so far: exp2(-inf - 0) = 0
+    m_run = m_new;
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s[r] = fast_exp2(__builtin_fmaf(s[r], c, -msub));
+      ps += s[r];
+    }
+    l_run = l_run * alpha + ps;
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+    // O^T += V^T P^T: the lane's half supplies key 8*q4 + 4*g + t on both operand sides
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+        o[db] = mfma_f32(lv[key * RS + 32 * db + lq], s[r], o[db]);
+      }
+  }
+
+  const float l_tot = xhalf_sum(l_run);
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (row < a.M) {
+    float* op = reinterpret_cast<float*>(a.o) + b * a.o_bs + h * a.o_hs + int64_t(row) * a.o_rs;
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d0 = 32 * db + 8 * q4 + 4 * g;
+        if (d0 >= D) continue;
+        const f32x4 x = {o[db][4 * q4] * inv, o[db][4 * q4 + 1] * inv, o[db][4 * q4 + 2] * inv, o[db][4 * q4 + 3] * inv};
+        *reinterpret_cast<f32x4*>(op + d0) = x;
+      }
+    if (g == 0) a.lse[(int64_t(b) * a.H + h) * a.M + row] = l_tot > 0.f ? m_run + fast_log2(l_tot) : -INFINITY;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int D, bool CAUSAL, bool DOC>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void dq_f32_kernel(const KArgs a) {
+  constexpr int RS = D + 1, KS2 = D / 2, DBN = (D + 31) / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* lk = reinterpret_cast<float*>(smem);
+  float* lv = lk + kRows * RS;
+  int* lid = reinterpret_cast<int*>(lv + kRows * RS);
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lq = lane & 31, g = lane >> 5;
+  const int BH = a.B * a.H;
+  const int nQt = (a.M + 127) / 128;
+  const int tile = nQt - 1 - blockIdx.x / BH;
+  const int bh = blockIdx.x % BH, b = bh / a.H, h = bh % a.H, hk = h / a.G;
+  const int m0 = tile * 128, mw = m0 + wave * 32;
+  const int row = mw + lq, rowc = min(row, a.M - 1);
+
+  const float* qp = reinterpret_cast<const float*>(a.q) + b * a.q_bs + h * a.q_hs + int64_t(rowc) * a.q_rs;
+  const float* dop = reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs + int64_t(rowc) * a.do_rs;
+  const float* kp = reinterpret_cast<const float*>(a.k) + b * a.k_bs + hk * a.k_hs;
+  const float* vp = reinterpret_cast<const float*>(a.v) + b * a.v_bs + hk * a.v_hs;
+  const int* ekp = DOC ? a.ek32 + b * a.ek_bs + h * a.ek_hs : nullptr;
+
+  const float c = a.scale_log2e;
+  float qreg[KS2], doreg[KS2];
+#pragma unroll
+  for (int s = 0; s < KS2; ++s) { qreg[s] = qp[2 * s + g]; doreg[s] = dop[2 * s + g]; }
+  float L_i = a.lse[(int64_t(b) * a.H + h) * a.M + rowc];
+  if (L_i == -INFINITY) L_i = INFINITY;   // row without any kept key: P = exp2(-inf) = 0
+  const float delta_i = a.delta[(int64_t(b) * a.H + h) * a.M + rowc];
+  const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
+  const bool glob_i = eq_i >= 0;
+  const int lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;
+  const int w_last = min(mw + 31, a.M - 1);
+  const int w_lim = CAUSAL ? min(a.gap + w_last, a.N - 1) : a.N - 1;
+  int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
+  if (DOC) {
+    const bool live = row < a.M;
+    w_lo = half_min(live && !glob_i ? eq_i : 0x7fffffff);
+    w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
+    w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
+  }
+  const int n_end = CAUSAL ? min(a.N, a.gap + min(m0 + 127, a.M - 1) + 1) : a.N;
+  const int nkt = (n_end + kRows - 1) / kRows;
+
+  f32x16 acc[DBN];
+#pragma unroll
+  for (int db = 0; db < DBN; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+
+  TileRegs<D> rk, rv;
+  int rid = 0;
+  rk.load(kp, a.k_rs, 0, a.N);
+  rv.load(vp, a.v_rs, 0, a.N);
+  if (DOC && threadIdx.x < kRows) rid = ekp[min((int)threadIdx.x, a.N - 1)];
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int n0 = kt * kRows;
+    __syncthreads();
+    rk.store(lk);
+    rv.store(lv);
+    if (DOC && threadIdx.x < kRows) lid[threadIdx.x] = rid;
+    __syncthreads();
+    if (kt + 1 < nkt) {
+      rk.load(kp, a.k_rs, n0 + kRows, a.N);
+      rv.load(vp, a.v_rs, n0 + kRows, a.N);
+      if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
+    }
+    bool skip = mw >= a.M || n0 > w_lim;
+    if (DOC && !skip) {
+      const bool kv = n0 + lq < a.N;
+      const int id = lid[lq];
+      const int k_lo = half_min(kv ? id : 0x7fffffff), k_hi = half_max(kv ? id : (int)0x80000000);
+      skip = !doc_may_keep(w_lo, w_hi, w_glob, k_lo, k_hi);
+    }
+    if (skip) continue;
+
+    f32x16 s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+    for (int st = 0; st < KS2; ++st) {
+      s = mfma_f32(lk[lq * RS + 2 * st + g], qreg[st], s);
+      dp = mfma_f32(lv[lq * RS + 2 * st + g], doreg[st], dp);
+    }
+    // dS = P (dP - delta); masked pairs -> 0 (a select, so an overflowed exponential of a masked pair is harmless)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = fast_exp2(__builtin_fmaf(s[r], c, -L_i)) * (dp[r] - delta_i);
+    mask_lim(s, lim_i - n0 - 4 * g, 0.f);
+    if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, 0.f);
+    // dQ^T += K^T dS^T
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+        acc[db] = mfma_f32(lk[key * RS + 32 * db + lq], s[r], acc[db]);
+      }
+  }
+
+  if (row < a.M) {
+    float* dqp = reinterpret_cast<float*>(a.dq) + b * a.dq_bs + h * a.dq_hs + int64_t(row) * a.dq_rs;
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d0 = 32 * db + 8 * q4 + 4 * g;
+        if (d0 >= D) continue;
+        const f32x4 x = {acc[db][4 * q4] * a.scale, acc[db][4 * q4 + 1] * a.scale, acc[db][4 * q4 + 2] * a.scale,
+                         acc[db][4 * q4 + 3] * a.scale};
+        *reinterpret_cast<f32x4*>(dqp + d0) = x;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int D, bool CAUSAL, bool DOC>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void dkdv_f32_kernel(const KArgs a) {
+  constexpr int RS = D + 1, KS2 = D / 2, DBN = (D + 31) / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* lqt = reinterpret_cast<float*>(smem);
+  float* ldo = lqt + kRows * RS;
+  float* laux = ldo + kRows * RS;               // [LSE | delta | eq] x 32
+  const int* leq = reinterpret_cast<const int*>(laux + 2 * kRows);
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lq = lane & 31, g = lane >> 5;
+  const int BHk = a.B * a.Hk;
+  const int kt = blockIdx.x / BHk;               // causal: the first keys are seen by the most rows: first
+  const int bhk = blockIdx.x % BHk, b = bhk / a.Hk, hk = bhk % a.Hk;
+  const int n0 = kt * 128, nw = n0 + wave * 32;
+  const int key = nw + lq, keyc = min(key, a.N - 1);
+
+  const float* kp = reinterpret_cast<const float*>(a.k) + b * a.k_bs + hk * a.k_hs + int64_t(keyc) * a.k_rs;
+  const float* vp = reinterpret_cast<const float*>(a.v) + b * a.v_bs + hk * a.v_hs + int64_t(keyc) * a.v_rs;
+  float kreg[KS2], vreg[KS2];   // B operands of S = Q K^T and dP = dO V^T: K[key][2*s + g], V[key][2*s + g]
+#pragma unroll
+  for (int s = 0; s < KS2; ++s) { kreg[s] = kp[2 * s + g]; vreg[s] = vp[2 * s + g]; }
+  const float c = a.scale_log2e;
+  // rows that may see this lane's key: [row_lo, row_lo + row_span)
+  const int row_lo = CAUSAL ? max(0, key - a.gap) : 0;
+  const unsigned row_span = key < a.N ? (unsigned)(a.M - row_lo) : 0u;
+  const int mt0 = CAUSAL ? max(0, n0 - a.gap) / kRows : 0;
+  const int nMt = (a.M + kRows - 1) / kRows;
+
+  f32x16 dv[DBN], dk[DBN];
+#pragma unroll
+  for (int db = 0; db < DBN; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dv[db][r] = 0.f; dk[db][r] = 0.f; }
+
+  for (int gi = 0; gi < a.G; ++gi) {
+    const int h = hk * a.G + gi;
+    const float* qp = reinterpret_cast<const float*>(a.q) + b * a.q_bs + h * a.q_hs;
+    const float* dop = reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs;
+    const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
+    const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+    const int* eqp = DOC ? a.eq32 + b * a.eq_bs + h * a.eq_hs : nullptr;
+    int ek_j = 0, wk_lo = 0, wk_hi = 0;
+    if (DOC) {
+      ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
+      wk_lo = half_min(key < a.N ? ek_j : 0x7fffffff);
+      wk_hi = half_max(key < a.N ? ek_j : (int)0x80000000);
+    }
+    // one auxiliary value per thread of the first three groups of 32: LSE, delta, eq of a tile row
+    auto aux_load = [&](int m0) -> float {
+      const int r = min(m0 + (int)(threadIdx.x & 31), a.M - 1);
+      const int which = threadIdx.x >> 5;
+      if (which == 0) return lsep[r];
+      if (which == 1) return delp[r];
+      if (which == 2 && DOC) return __int_as_float(eqp[r]);
+      return 0.f;
+    };
+    TileRegs<D> rq, rdo;
+    float raux = 0.f;
+    if (mt0 < nMt) {
+      rq.load(qp, a.q_rs, mt0 * kRows, a.M);
+      rdo.load(dop, a.do_rs, mt0 * kRows, a.M);
+      if (threadIdx.x < 3 * kRows) raux = aux_load(mt0 * kRows);
+    }
+    for (int mt = mt0; mt < nMt; ++mt) {
+      const int m0 = mt * kRows;
+      __syncthreads();
+      rq.store(lqt);
+      rdo.store(ldo);
+      if (threadIdx.x < 3 * kRows) laux[threadIdx.x] = raux;
+      __syncthreads();
+      if (mt + 1 < nMt) {
+        rq.load(qp, a.q_rs, m0 + kRows, a.M);
+        rdo.load(dop, a.do_rs, m0 + kRows, a.M);
+        if (threadIdx.x < 3 * kRows) raux = aux_load(m0 + kRows);
+      }
+      bool skip = nw >= a.N || (CAUSAL && a.gap + min(m0 + kRows - 1, a.M - 1) < nw);
+      if (DOC && !skip) {
+        const bool rv_ = m0 + lq < a.M;
+        const int id = leq[lq];
+        const bool loc = rv_ && id < 0;
+        const int q_lo = half_min(loc ? id : 0x7fffffff), q_hi = half_max(loc ? id : (int)0x80000000);
+        const int q_glob = __builtin_amdgcn_ballot_w64(rv_ && id >= 0) != 0;
+        skip = !doc_may_keep(q_lo, q_hi, q_glob, wk_lo, wk_hi);
+      }
+      if (skip) continue;
+
+      f32x16 x, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { x[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+      for (int st = 0; st < KS2; ++st) {
+        x = mfma_f32(lqt[lq * RS + 2 * st + g], kreg[st], x);
+        dp = mfma_f32(ldo[lq * RS + 2 * st + g], vreg[st], dp);
+      }
+      // lane = key, register 4*q4 + t = row 8*q4 + 4*g + t of the tile
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int i0 = 8 * q4 + 4 * g;
+        const f32x4 Lv = *reinterpret_cast<const f32x4*>(laux + i0);
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(laux + kRows + i0);
+        const i32x4 eqv = *reinterpret_cast<const i32x4*>(leq + i0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          bool keep = (unsigned)(m0 + i0 + t - row_lo) < row_span;
+          if (DOC) keep = keep && (eqv[t] >= 0 || eqv[t] == ek_j);
+          const float p = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
+          x[4 * q4 + t] = keep ? p : 0.f;
+          dp[4 * q4 + t] = keep ? p * (dp[4 * q4 + t] - dl[t]) : 0.f;
+        }
+      }
+      // dV^T += dO^T P, dK^T += Q^T dS
+#pragma unroll
+      for (int db = 0; db < DBN; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qr = 8 * (r >> 2) + 4 * g + (r & 3);
+          dv[db] = mfma_f32(ldo[qr * RS + 32 * db + lq], x[r], dv[db]);
+          dk[db] = mfma_f32(lqt[qr * RS + 32 * db + lq], dp[r], dk[db]);
+        }
+    }
+  }
+
+  if (key < a.N) {
+    float* dvp = reinterpret_cast<float*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs;
+    float* dkp = reinterpret_cast<float*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
+#pragma unroll
+    for (int db = 0; db < DBN; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d0 = 32 * db + 8 * q4 + 4 * g;
+        if (d0 >= D) continue;
+        const f32x4 xv = {dv[db][4 * q4], dv[db][4 * q4 + 1], dv[db][4 * q4 + 2], dv[db][4 * q4 + 3]};
+        const f32x4 xk = {dk[db][4 * q4] * a.scale, dk[db][4 * q4 + 1] * a.scale, dk[db][4 * q4 + 2] * a.scale,
+                          dk[db][4 * q4 + 3] * a.scale};
+        *reinterpret_cast<f32x4*>(dvp + d0) = xv;
+        *reinterpret_cast<f32x4*>(dkp + d0) = xk;
+      }
+  }
+}
+
+// delta[b,h,m] = sum_d O[b,h,m,d] * dO[b,h,m,d]; D/4 lanes per row, 16-byte loads.
+template <int D>
+__global__ __launch_bounds__(kThreads) void delta_f32_kernel(const KArgs a) {
+  constexpr int LPR = D / 4, RPB = kThreads / LPR;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int row = blockIdx.x * RPB + threadIdx.x / LPR;
+  const int cc = threadIdx.x % LPR;
+  float acc = 0.f;
+  if (row < a.M) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.o) + b * a.o_bs + h * a.o_hs +
+                                                    int64_t(row) * a.o_rs + cc * 4);
+    const f32x4 y = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs +
+                                                    int64_t(row) * a.do_rs + cc * 4);
+    acc = x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+  }
+#pragma unroll
+  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
+  if (cc == 0 && row < a.M) a.delta[(int64_t(b) * a.H + h) * a.M + row] = acc;
+}
+
+enum { kFwd, kDq, kDkdv };
+
+template <int WHICH, int D, bool CAUSAL, bool DOC>
+int launch_one(const KArgs& a, hipStream_t s) {
+  auto kern = WHICH == kFwd ? fwd_f32_kernel<D, CAUSAL, DOC> : WHICH == kDq ? dq_f32_kernel<D, CAUSAL, DOC>
+                                                                            : dkdv_f32_kernel<D, CAUSAL, DOC>;
+  const int blocks = WHICH == kDkdv ? ((a.N + 127) / 128) * a.B * a.Hk : ((a.M + 127) / 128) * a.B * a.H;
+  static bool lds_allowed[64] = {};   // per kernel instantiation and device
+  if (int e = allow_lds(kern, lds_bytes<D>(), lds_allowed)) return e;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreads), lds_bytes<D>(), s, a);
+  return (int)hipGetLastError();
+}
+
+template <int WHICH, int D>
+int launch_cd(const KArgs& a, bool causal, bool doc, hipStream_t s) {
+  if (causal) return doc ? launch_one<WHICH, D, true, true>(a, s) : launch_one<WHICH, D, true, false>(a, s);
+  return doc ? launch_one<WHICH, D, false, true>(a, s) : launch_one<WHICH, D, false, false>(a, s);
+}
+
+template <int WHICH>
+int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) {
+  switch (D) {
+    case 128: return launch_cd<WHICH, 128>(a, causal, doc, s);
+    case 64: return launch_cd<WHICH, 64>(a, causal, doc, s);
+    case 32: return launch_cd<WHICH, 32>(a, causal, doc, s);
+    case 16: return launch_cd<WHICH, 16>(a, causal, doc, s);
+    default: return -1;
+  }
+}
+
+}  // namespace
+
+int launch_fwd_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) { return launch_d<kFwd>(a, D, causal, doc, s); }
+int launch_bwd_dq_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) { return launch_d<kDq>(a, D, causal, doc, s); }
+int launch_bwd_dkdv_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) { return launch_d<kDkdv>(a, D, causal, doc, s); }
+
+int launch_bwd_delta_f32(const KArgs& a, int D, hipStream_t s) {
+  const int BH = a.B * a.H;
+  switch (D) {
+    case 128: hipLaunchKernelGGL((delta_f32_kernel<128>), dim3((a.M + 7) / 8, BH), dim3(kThreads), 0, s, a); break;
+    case 64: hipLaunchKernelGGL((delta_f32_kernel<64>), dim3((a.M + 15) / 16, BH), dim3(kThreads), 0, s, a); break;
+    case 32: hipLaunchKernelGGL((delta_f32_kernel<32>), dim3((a.M + 31) / 32, BH), dim3(kThreads), 0, s, a); break;
+    case 16: hipLaunchKernelGGL((delta_f32_kernel<16>), dim3((a.M + 63) / 64, BH), dim3(kThreads), 0, s, a); break;
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace fa

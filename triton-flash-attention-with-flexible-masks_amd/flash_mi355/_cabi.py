@@ -16,6 +16,7 @@ FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
 FA_DTYPE_BF16 = 0
 FA_DTYPE_FP16 = 1
+FA_DTYPE_FP32 = 2
 FA_IDTYPE_I32 = 0
 FA_IDTYPE_I64 = 1
 

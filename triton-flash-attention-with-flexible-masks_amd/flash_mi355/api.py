@@ -17,7 +17,7 @@ from . import _cabi
 SCORE_FUNC_MODE0_NOPE = 0  # flash_triton.py:20
 SCORE_FUNC_MODE1_DOC = 1   # flash_triton.py:22
 
-_DTYPES = {torch.bfloat16: _cabi.FA_DTYPE_BF16, torch.float16: _cabi.FA_DTYPE_FP16}
+_DTYPES = {torch.bfloat16: _cabi.FA_DTYPE_BF16, torch.float16: _cabi.FA_DTYPE_FP16, torch.float32: _cabi.FA_DTYPE_FP32}
 _ID_DTYPES = {torch.int32: _cabi.FA_IDTYPE_I32, torch.int64: _cabi.FA_IDTYPE_I64}
 
 
@@ -27,8 +27,9 @@ def maybe_contiguous(x):
 
 
 def _aligned(x):
-    """16-byte aligned base and outer strides that are multiples of 8 elements."""
-    ok = x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+    """16-byte aligned base and outer strides that are multiples of 16 bytes."""
+    per16 = 16 // x.element_size()
+    ok = x.data_ptr() % 16 == 0 and all(s % per16 == 0 for s in x.stride()[:-1])
     return x if ok else x.contiguous()
 
 
@@ -131,7 +132,7 @@ class _Impl:
         assert score_func_mode in (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC), "unknown score_func_mode"
         assert q.is_cuda and k.is_cuda and v.is_cuda, "flash_mi355 runs on the GPU only"
         assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, \
-            "q, k, v must share one of torch.bfloat16 / torch.float16"
+            "q, k, v must share one of torch.bfloat16 / torch.float16 / torch.float32"
         assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
         if score_func_mode != SCORE_FUNC_MODE0_NOPE:
             eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")

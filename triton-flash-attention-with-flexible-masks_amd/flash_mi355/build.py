@@ -20,7 +20,7 @@ INCLUDE = PKG_DIR.parent.parent / "include"
 LIB_PATH = PKG_DIR / "libflash_mi355.so"
 OBJ_DIR = PKG_DIR / "_obj"
 
-SOURCES = ["fa_api.hip", "fa_aux.hip", "fa_fwd.hip", "fa_bwd_dq.hip", "fa_bwd_dkdv.hip"]
+SOURCES = ["fa_api.hip", "fa_aux.hip", "fa_fwd.hip", "fa_bwd_dq.hip", "fa_bwd_dkdv.hip", "fa_f32.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
