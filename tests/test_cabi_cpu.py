@@ -71,6 +71,10 @@ def test_validate_codes():
     p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
     p = _good_params(buf); p.flags = 1; assert v(p) == -7
+    # fp32 tensors are accepted; their strides must be multiples of 16 bytes = 4 elements
+    p = _good_params(buf); p.dtype = _cabi.FA_DTYPE_FP32; assert v(p) == 0
+    p = _good_params(buf); p.dtype = _cabi.FA_DTYPE_FP32; p.q_stride[2] = 68; assert v(p) == 0
+    p = _good_params(buf); p.dtype = _cabi.FA_DTYPE_FP32; p.q_stride[2] = 66; assert v(p) == -5
 
 
 def test_workspace_size():
