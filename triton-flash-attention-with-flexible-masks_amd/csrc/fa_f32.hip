@@ -73,6 +73,29 @@ FA_DEV int half_max(int x) {
   return x;
 }
 
+// A run of N MFMAs whose A operands come from LDS: the operands are requested a chunk of CH ahead
+// of the MFMAs that consume them, in program order (left to itself the compiler puts a read, a
+// full wait and its MFMAs back to back).  rd(i) reads operand i, mm(i, a) issues MFMA i.
+template <int N, int CH, typename RD, typename MM>
+FA_DEV void pipelined(RD&& rd, MM&& mm) {
+  static_assert(N % CH == 0, "chunking");
+  float buf[2][CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) buf[0][i] = rd(i);
+#pragma unroll
+  for (int c = 0; c < N / CH; ++c) {
+    if (c + 1 < N / CH) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) buf[(c + 1) & 1][i] = rd((c + 1) * CH + i);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) mm(c * CH + i, buf[c & 1][i]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+constexpr int kChunk = 8;
+
 template <int D>
 constexpr size_t lds_bytes() { return size_t(2 * kRows * (D + 1) + 4 * kRows + 64) * 4; }
 
@@ -162,8 +185,8 @@ void fwd_f32_kernel(const KArgs a) {
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-    for (int st = 0; st < KS2; ++st) s = mfma_f32(lk[lq * RS + 2 * st + g], qreg[st], s);
+    pipelined<KS2, kChunk>([&](int i) __attribute__((always_inline)) { return lk[lq * RS + 2 * i + g]; },
+                           [&](int i, float x) __attribute__((always_inline)) { s = mfma_f32(x, qreg[i], s); });
     mask_lim(s, lim_i - n0 - 4 * g, -INFINITY);
     if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, -INFINITY);
 
@@ -187,13 +210,12 @@ void fwd_f32_kernel(const KArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
     // O^T += V^T P^T: the lane's half supplies key 8*q4 + 4*g + t on both operand sides
-#pragma unroll
-    for (int db = 0; db < DBN; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-        o[db] = mfma_f32(lv[key * RS + 32 * db + lq], s[r], o[db]);
-      }
+    pipelined<16 * DBN, kChunk>(
+        [&](int i) __attribute__((always_inline)) {
+          const int r = i % 16, key = 8 * (r >> 2) + 4 * g + (r & 3);
+          return lv[key * RS + 32 * (i / 16) + lq];
+        },
+        [&](int i, float x) __attribute__((always_inline)) { o[i / 16] = mfma_f32(x, s[i % 16], o[i / 16]); });
   }
 
   const float l_tot = xhalf_sum(l_run);
@@ -296,24 +318,24 @@ void dq_f32_kernel(const KArgs a) {
     f32x16 s, dp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-    for (int st = 0; st < KS2; ++st) {
-      s = mfma_f32(lk[lq * RS + 2 * st + g], qreg[st], s);
-      dp = mfma_f32(lv[lq * RS + 2 * st + g], doreg[st], dp);
-    }
+    pipelined<2 * KS2, kChunk>(
+        [&](int i) __attribute__((always_inline)) { return ((i & 1) ? lv : lk)[lq * RS + 2 * (i / 2) + g]; },
+        [&](int i, float x) __attribute__((always_inline)) {
+          if (i & 1) dp = mfma_f32(x, doreg[i / 2], dp);
+          else s = mfma_f32(x, qreg[i / 2], s);
+        });
     // dS = P (dP - delta); masked pairs -> 0 (a select, so an overflowed exponential of a masked pair is harmless)
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = fast_exp2(__builtin_fmaf(s[r], c, -L_i)) * (dp[r] - delta_i);
     mask_lim(s, lim_i - n0 - 4 * g, 0.f);
     if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, 0.f);
     // dQ^T += K^T dS^T
-#pragma unroll
-    for (int db = 0; db < DBN; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-        acc[db] = mfma_f32(lk[key * RS + 32 * db + lq], s[r], acc[db]);
-      }
+    pipelined<16 * DBN, kChunk>(
+        [&](int i) __attribute__((always_inline)) {
+          const int r = i % 16, key = 8 * (r >> 2) + 4 * g + (r & 3);
+          return lk[key * RS + 32 * (i / 16) + lq];
+        },
+        [&](int i, float x) __attribute__((always_inline)) { acc[i / 16] = mfma_f32(x, s[i % 16], acc[i / 16]); });
   }
 
   if (row < a.M) {
@@ -423,11 +445,12 @@ void dkdv_f32_kernel(const KArgs a) {
       f32x16 x, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { x[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-      for (int st = 0; st < KS2; ++st) {
-        x = mfma_f32(lqt[lq * RS + 2 * st + g], kreg[st], x);
-        dp = mfma_f32(ldo[lq * RS + 2 * st + g], vreg[st], dp);
-      }
+      pipelined<2 * KS2, kChunk>(
+          [&](int i) __attribute__((always_inline)) { return ((i & 1) ? ldo : lqt)[lq * RS + 2 * (i / 2) + g]; },
+          [&](int i, float v_) __attribute__((always_inline)) {
+            if (i & 1) dp = mfma_f32(v_, vreg[i / 2], dp);
+            else x = mfma_f32(v_, kreg[i / 2], x);
+          });
       // lane = key, register 4*q4 + t = row 8*q4 + 4*g + t of the tile
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
@@ -445,14 +468,16 @@ void dkdv_f32_kernel(const KArgs a) {
         }
       }
       // dV^T += dO^T P, dK^T += Q^T dS
-#pragma unroll
-      for (int db = 0; db < DBN; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int qr = 8 * (r >> 2) + 4 * g + (r & 3);
-          dv[db] = mfma_f32(ldo[qr * RS + 32 * db + lq], x[r], dv[db]);
-          dk[db] = mfma_f32(lqt[qr * RS + 32 * db + lq], dp[r], dk[db]);
-        }
+      pipelined<32 * DBN, kChunk>(
+          [&](int i) __attribute__((always_inline)) {
+            const int r = (i / 2) % 16, qr = 8 * (r >> 2) + 4 * g + (r & 3);
+            return ((i & 1) ? lqt : ldo)[qr * RS + 32 * (i / 32) + lq];
+          },
+          [&](int i, float v_) __attribute__((always_inline)) {
+            const int r = (i / 2) % 16, db = i / 32;
+            if (i & 1) dk[db] = mfma_f32(v_, dp[r], dk[db]);
+            else dv[db] = mfma_f32(v_, x[r], dv[db]);
+          });
     }
   }
 
