@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 1
+#define FA_ABI_VERSION 2
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
@@ -104,6 +104,14 @@ typedef struct fa_params {
   int32_t id_dtype;       /* FA_IDTYPE_* (eq, ek) */
   float   sm_scale;
   int32_t flags;          /* reserved, must be 0 */
+  /* Two more causal masks on the same machinery (no counterpart in the reference, whose README.md:17-18
+     names such masks as the extension point); 0 = off; both need causal != 0 and exclude each other:
+       window > 0 : sliding window -- row i sees only the last `window` keys up to its diagonal:
+                    keep additionally needs j > max(0,N-M) + i - window
+       prefix > 0 : prefix-LM -- the first `prefix` keys are seen by every row:
+                    the causal term becomes (max(0,N-M) + i >= j) || (j < prefix)                     */
+  int32_t window;
+  int32_t prefix;
 } fa_params;
 
 /* ABI version of the loaded library (== FA_ABI_VERSION of the header it was built from). */
@@ -135,8 +143,8 @@ uint64_t fa_workspace_plan_bytes(const fa_params* p);
 /* Mask engine: normalise eq/ek to int32 and build per-tile id summaries
    into p->workspace.  Must be enqueued before fa_fwd / fa_bwd_* on the same
    stream whenever score_mode != 0.  The same workspace serves forward and backward.
-   The plan depends on the ids, the sizes AND on `causal` (key ranges are narrowed with the
-   causal bound): plan again when any of them changes.  The workspace also holds the scratch
+   The plan depends on the ids, the sizes AND on `causal` and `prefix` (key ranges are narrowed with
+   the causal bound): plan again when any of them changes.  The workspace also holds the scratch
    of the tiles whose key range is split over several workgroups, so two launches that share a
    workspace must be ordered on one stream. */
 int fa_mask_plan(const fa_params* p, void* stream);

@@ -71,6 +71,12 @@ def test_validate_codes():
     p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
     p = _good_params(buf); p.flags = 1; assert v(p) == -7
+    # sliding window / prefix: causal only, not both, not negative
+    p = _good_params(buf); p.window = 64; assert v(p) == 0
+    p = _good_params(buf); p.prefix = 64; assert v(p) == 0
+    p = _good_params(buf); p.window = 64; p.prefix = 8; assert v(p) == -7
+    p = _good_params(buf); p.window = -1; assert v(p) == -7
+    p = _good_params(buf); p.M, p.N, p.causal, p.window = 256, 128, 0, 16; assert v(p) == -7
     # fp32 tensors are accepted; their strides must be multiples of 16 bytes = 4 elements
     p = _good_params(buf); p.dtype = _cabi.FA_DTYPE_FP32; assert v(p) == 0
     p = _good_params(buf); p.dtype = _cabi.FA_DTYPE_FP32; p.q_stride[2] = 68; assert v(p) == 0
@@ -136,5 +142,8 @@ def test_drop_in_module_name():
     assert (flash_triton.SCORE_FUNC_MODE0_NOPE, flash_triton.SCORE_FUNC_MODE1_DOC) == (0, 1)
     import inspect
     sig = inspect.signature(flash_triton.attention)
-    assert list(sig.parameters) == ["q", "k", "v", "causal", "sm_scale", "eq", "ek", "score_func_mode"]
-    assert [p.default for p in sig.parameters.values()][3:] == [False, None, None, None, 0]
+    pos = [n for n, p in sig.parameters.items() if p.kind == p.POSITIONAL_OR_KEYWORD]
+    assert pos == ["q", "k", "v", "causal", "sm_scale", "eq", "ek", "score_func_mode"]   # flash_triton.py:640
+    extra = {n: p for n, p in sig.parameters.items() if n not in pos}
+    assert all(p.kind == p.KEYWORD_ONLY and p.default == 0 for p in extra.values())     # additions stay out of the way
+    assert [sig.parameters[n].default for n in pos][3:] == [False, None, None, None, 0]

@@ -28,7 +28,7 @@ def _ids(rng, B, H, L, kind):
 
 
 def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
-              id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE):
+              id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE, window=0, prefix=0):
     from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
     from oracle import attention_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -47,7 +47,8 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
         else:
             ek = torch.from_numpy(_ids(rng, B, H, N, ids_kind)).to(id_dtype)[:, None, :].expand(B, H, N)
         eq = ek[:, :, N - M:]  # queries are the last M positions (self-attention when M == N)
-    print(f"case B{B} H{H}/{Hk} M{M} N{N} D{D} {dtype} causal={causal} doc={doc} seed={seed} ids={ids_kind}", flush=True)
+    print(f"case B{B} H{H}/{Hk} M{M} N{N} D{D} {dtype} causal={causal} doc={doc} seed={seed} ids={ids_kind} "
+          f"window={window} prefix={prefix}", flush=True)
 
     qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
     eqd = eq.cuda() if eq is not None else None
@@ -55,9 +56,11 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
     if eqd is not None and not per_head_ids:
         eqd = eq[:, :1].contiguous().cuda().expand(B, H, M)
         ekd = ek[:, :1].contiguous().cuda().expand(B, H, N)
-    out, lse = attention_with_lse(qd.detach(), kd.detach(), vd.detach(), causal, sm_scale, eqd, ekd, mode)
+    out, lse = attention_with_lse(qd.detach(), kd.detach(), vd.detach(), causal, sm_scale, eqd, ekd, mode,
+                                  window=window, prefix=prefix)
     torch.cuda.synchronize()
-    ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, sm_scale, eq, ek, mode)
+    ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, sm_scale, eq, ek, mode,
+                                                                   window=window, prefix=prefix)
     # rows without any kept key: O = 0, LSE = -inf on both sides
     dead = torch.isinf(ref_lse)
     assert torch.equal(torch.isinf(lse.cpu()), dead)
@@ -68,7 +71,7 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
     assert o_err <= tol_o, f"O err {o_err}"
     if not check_bwd:
         return
-    out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode)
+    out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode, window=window, prefix=prefix)
     out2.backward(do.cuda())
     torch.cuda.synchronize()
     assert torch.equal(out2.detach(), out)
@@ -460,3 +463,59 @@ def test_fp32_tensors(case):
 def test_fp32_all_global_and_all_local_ids():
     _run_case(1, 2, 2, 160, 160, 64, torch.float32, True, True, seed=6, ids_kind="allglobal", tol_o=TOL_F32, tol_lse=TOL_F32)
     _run_case(1, 2, 2, 160, 160, 64, torch.float32, False, True, seed=6, ids_kind="alllocal", tol_o=TOL_F32, tol_lse=TOL_F32)
+
+
+# Sliding window and prefix-LM (causal masks the library adds; no counterpart in the reference):
+# checked against the oracle's closed form like every other case.
+BAND_CASES = [
+    # B, H, Hk, M, N, D, dtype, doc, window, prefix
+    (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 100, 0),
+    (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 1, 0),
+    (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 64, 0),
+    (1, 2, 2, 300, 300, 64, torch.bfloat16, True, 77, 0),      # window + ids, ragged
+    (1, 4, 2, 200, 456, 128, torch.float16, True, 130, 0),     # window + ids, rectangular, grouped-query
+    (1, 2, 2, 2048, 2048, 64, torch.bfloat16, False, 256, 0),  # many key tiles before the window
+    (1, 2, 2, 2048, 2048, 128, torch.bfloat16, True, 300, 0),
+    (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 0, 200),
+    (1, 2, 2, 512, 512, 64, torch.bfloat16, False, 0, 1),
+    (1, 2, 2, 300, 300, 128, torch.bfloat16, True, 0, 150),    # prefix + ids
+    (1, 2, 2, 128, 512, 128, torch.float16, True, 0, 450),     # prefix reaching past the first rows' diagonal, rectangular
+    (1, 2, 2, 256, 256, 32, torch.bfloat16, True, 0, 256),     # everything is prefix
+    (1, 2, 2, 256, 256, 16, torch.bfloat16, True, 33, 0),
+    (1, 2, 2, 333, 333, 64, torch.float32, True, 50, 0),
+    (1, 2, 2, 333, 333, 128, torch.float32, False, 0, 100),
+    (1, 4, 2, 100, 260, 32, torch.float32, True, 0, 200),
+]
+
+
+@pytest.mark.parametrize("case", BAND_CASES, ids=lambda c: "B%d-H%d_%d-M%d-N%d-D%d-%s-d%d-w%d-p%d" % (
+    c[0], c[1], c[2], c[3], c[4], c[5], str(c[6]).split(".")[-1], c[7], c[8], c[9]))
+def test_sliding_window_and_prefix(case):
+    B, H, Hk, M, N, D, dtype, doc, window, prefix = case
+    tol = TOL_F32 if dtype == torch.float32 else TOL_O
+    _run_case(B, H, Hk, M, N, D, dtype, True, doc, seed=77, window=window, prefix=prefix, tol_o=tol,
+              tol_lse=TOL_F32 if dtype == torch.float32 else TOL_LSE)
+
+
+def test_window_and_prefix_mask_bit_exact():
+    from flash_mi355 import mask_dump, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    rng = np.random.default_rng(9)
+    for (B, H, M, N) in [(1, 2, 200, 200), (1, 2, 77, 333)]:
+        ek = torch.from_numpy(np.stack([_ids(rng, B, H, N, "uniform") for _ in range(H)], axis=1))
+        eq = torch.from_numpy(np.stack([_ids(rng, B, H, M, "uniform") for _ in range(H)], axis=1))
+        for kw in ({"window": 1}, {"window": 40}, {"window": 1000}, {"prefix": 1}, {"prefix": 90}, {"prefix": 1000}):
+            got = mask_dump(B, H, M, N, True, eq.cuda(), ek.cuda(), SCORE_FUNC_MODE1_DOC, **kw).cpu().numpy()
+            ref = np.broadcast_to(O.keep_mask(M, N, True, eq.numpy(), ek.numpy(), 1, **kw), (B, H, M, N))
+            assert np.array_equal(got, ref), kw
+            got = mask_dump(B, H, M, N, True, **kw).cpu().numpy()
+            assert np.array_equal(got, np.broadcast_to(O.keep_mask(M, N, True, **kw), (B, H, M, N))), kw
+
+
+def test_window_needs_causal():
+    from flash_mi355 import attention
+    q = torch.randn(1, 1, 64, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        attention(q, q, q, False, window=8)
+    with pytest.raises(AssertionError):
+        attention(q, q, q, True, window=8, prefix=8)

@@ -233,3 +233,53 @@ def test_eager_cpu_path_matches_closed_form():
     got = O.eager_attention_cpu(q, k, v, True, keep)
     ref, _ = O.attention_closed_form(q, k, v, True, None, eq, ek, 1)
     assert torch.allclose(got, ref, atol=1e-5)
+
+
+# ------------------------------------------------------------------ sliding window / prefix-LM
+@pytest.mark.parametrize("M,N", [(9, 9), (5, 12), (1, 6)])
+def test_window_and_prefix_masks_brute_force(M, N):
+    """The two causal variants the library adds, element by element in Python loops, alone and with
+    ids, square and bottom-right aligned."""
+    rng = np.random.default_rng(M * 31 + N)
+    eq, ek = _ids(rng, 1, 2, M), _ids(rng, 1, 2, N)
+    gap = max(0, N - M)
+    for window, prefix in [(1, 0), (3, 0), (N, 0), (N + 5, 0), (0, 1), (0, 4), (0, N), (0, N + 3)]:
+        plain = np.broadcast_to(O.keep_mask(M, N, True, window=window, prefix=prefix), (1, 1, M, N))
+        doc = np.broadcast_to(O.keep_mask(M, N, True, eq, ek, 1, window=window, prefix=prefix), (1, 2, M, N))
+        for i in range(M):
+            for j in range(N):
+                c = gap + i >= j or (prefix and j < prefix)
+                if window:
+                    c = c and j > gap + i - window
+                assert plain[0, 0, i, j] == bool(c)
+                for h in range(2):
+                    assert doc[0, h, i, j] == bool(c and (eq[0, h, i] >= 0 or eq[0, h, i] == ek[0, h, j]))
+
+
+def test_window_and_prefix_special_cases():
+    L = 10
+    causal = O.keep_mask(L, L, True)
+    assert np.array_equal(O.keep_mask(L, L, True, window=L), causal)          # a window as long as the row: no effect
+    assert np.array_equal(O.keep_mask(L, L, True, window=1)[0, 0], np.eye(L, dtype=bool))   # only the diagonal
+    assert np.array_equal(O.keep_mask(L, L, True, window=3)[0, 0], np.tril(np.ones((L, L), bool)) & ~np.tril(np.ones((L, L), bool), -3))
+    assert np.array_equal(O.keep_mask(L, L, True, prefix=0), causal)
+    assert O.keep_mask(L, L, True, prefix=L).all()                               # everything is prefix: no mask left
+    want = np.tril(np.ones((L, L), bool)); want[:4, :4] = True                   # textbook prefix-LM: bidirectional block + causal
+    assert np.array_equal(O.keep_mask(L, L, True, prefix=4)[0, 0], want)
+    with pytest.raises(AssertionError):
+        O.keep_mask(L, L, False, window=3)
+    with pytest.raises(AssertionError):
+        O.keep_mask(L, L, True, window=3, prefix=2)
+
+
+def test_closed_form_with_window_matches_sdpa():
+    """O with a sliding window / prefix against torch SDPA fed an independently built mask."""
+    g = torch.Generator().manual_seed(4)
+    B, H, M, N, D = 1, 2, 12, 20, 16
+    q, k, v = torch.randn(B, H, M, D, generator=g), torch.randn(B, H, N, D, generator=g), torch.randn(B, H, N, D, generator=g)
+    i = torch.arange(M)[:, None] + (N - M)
+    j = torch.arange(N)[None, :]
+    for kw, mask in (({"window": 5}, (i >= j) & (j > i - 5)), ({"prefix": 7}, (i >= j) | (j < 7))):
+        o, _ = O.attention_closed_form(q, k, v, True, None, **kw)
+        ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+        assert (o - ref).abs().max().item() < 1e-5

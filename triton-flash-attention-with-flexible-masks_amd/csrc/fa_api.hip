@@ -34,7 +34,7 @@ extern "C" const char* fa_error_string(int code) {
     case FA_ERR_SHAPE: return "inconsistent sizes (H % Hk != 0, causal with N < M, or a size <= 0)";
     case FA_ERR_ALIGN: return "pointers must be 16-byte aligned and outer strides multiples of 16 bytes";
     case FA_ERR_STRIDE: return "innermost stride must be 1";
-    case FA_ERR_MODE: return "unknown score mode, or doc mode without eq/ek";
+    case FA_ERR_MODE: return "unknown score mode, doc mode without eq/ek, or window / prefix without causal (or both)";
     case FA_ERR_WORKSPACE: return "workspace missing or too small";
     case FA_ERR_HIP: return "kernel launch failed";
     case FA_ERR_NOT_IMPLEMENTED: return "configuration not implemented";
@@ -51,6 +51,8 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
   if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC) return FA_ERR_MODE;
   if (p->flags != 0) return FA_ERR_MODE;
+  if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
+  if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     if (p->eq == nullptr || p->ek == nullptr) return FA_ERR_MODE;
     if (p->id_dtype != FA_IDTYPE_I32 && p->id_dtype != FA_IDTYPE_I64) return FA_ERR_DTYPE;
@@ -101,6 +103,8 @@ static KArgs make_args(const fa_params* p) {
   a.dv_bs = p->dv_stride[0]; a.dv_hs = p->dv_stride[1]; a.dv_rs = p->dv_stride[2];
   a.B = p->B; a.H = p->H; a.Hk = p->Hk; a.G = p->H / p->Hk; a.M = p->M; a.N = p->N;
   a.gap = p->N > p->M ? p->N - p->M : 0;  // flash_triton.py:521
+  a.win = p->window > 0 ? (p->window < 0x3fffffff ? p->window : 0x3fffffff) : 0x3fffffff;
+  a.pfx_m1 = p->prefix > 0 ? (p->prefix < p->N ? p->prefix : p->N) - 1 : -1;
   a.scale = p->sm_scale;
   a.scale_log2e = p->sm_scale * kLog2e;
   a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.peq = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
 // Step 3: one wave per 64 entries of the permuted order: id / row-index summary, and the range
 // [kfirst, klast] of key tiles the entry's rows can need (by the key summaries and the causal
 // bound), so that the compute kernels start their tile search in the right place.
-__global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal_gap,
+__global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal_gap, int kend_min,
                                                         const int* __restrict__ perm, const int* __restrict__ peq,
                                                         const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum,
                                                         int* __restrict__ sk_cnt, int n_sk) {
@@ -172,7 +172,8 @@ __global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs
   int kfirst = 0x7fffffff, klast = -1;
   if (H1 == HK1) {  // ids of both sides stored per the same heads: narrow the key range
     const IdSummary* ks = ksum + bh * nKs;
-    const int kend = causal_gap >= 0 ? min(nKs, (causal_gap + s.rmax) / kSumRows + 1) : nKs;
+    // kend_min: key tiles of a prefix that every row sees whatever its causal bound
+    const int kend = causal_gap >= 0 ? min(nKs, max((causal_gap + s.rmax) / kSumRows + 1, kend_min)) : nKs;
     for (int k0 = 0; k0 < kend; k0 += 64) {
       const int k = k0 + lane;
       bool cand = false;
@@ -226,7 +227,7 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     const int gap = p->N > p->M ? p->N - p->M : 0;
     hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
-                       p->causal ? gap : -1, perm, peq, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
+                       p->causal ? gap : -1, p->prefix > 0 ? ((p->prefix < p->N ? p->prefix : p->N) - 1) / kSumRows + 1 : 0, perm, peq, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
                        p->B * p->H * split_config(p->B, p->H, p->N, p->D).tiles);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(256) void mask_dump_kernel(const KArgs a, uint8_t* 
     eq_i = a.eq32[b * a.eq_bs + h * a.eq_hs + i];
     ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + j];
   }
-  out[(int64_t(bh) * a.M + i) * a.N + j] = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j) ? 1 : 0;
+  out[(int64_t(bh) * a.M + i) * a.N + j] = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1) ? 1 : 0;
 }
 
 int launch_mask_dump(const KArgs& a, bool causal, bool doc, uint8_t* out, hipStream_t s) {

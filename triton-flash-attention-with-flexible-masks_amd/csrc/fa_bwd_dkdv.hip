@@ -94,8 +94,10 @@ void bwd_dkdv_kernel(const KArgs a) {
   for (int ks = 0; ks < KS; ++ks) settle(frag[ks]);
   const float c = a.scale_log2e;
   // rows that may see this lane's key: [row_lo, row_lo + row_span)
-  const int row_lo = CAUSAL ? max(0, key - a.gap) : 0;
-  const unsigned row_span = key < a.N ? (unsigned)(a.M - row_lo) : 0u;
+  // (causal: from the diagonal on, or from row 0 for a key of the prefix; sliding window: `win` rows)
+  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - a.gap)) : 0;
+  const int row_hi = CAUSAL ? min(a.M - 1, key - a.gap + a.win - 1) : a.M - 1;
+  const unsigned row_span = (key < a.N && row_hi >= row_lo) ? (unsigned)(row_hi - row_lo + 1) : 0u;
 
   // per query head state (set at the top of the head loop)
   const float* lsep = nullptr;
@@ -552,7 +554,10 @@ void bwd_dkdv_kernel(const KArgs a) {
     ldO.init(reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs, a.do_rs, a.M);
     int gk_lo = 0, gk_hi = 0;   // id interval of the workgroup's 128 keys
     int nQtiles = (a.M + BQ - 1) / BQ;
-    int first = CAUSAL ? max(0, n0 - a.gap) / BQ : 0;
+    int first = CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - a.gap) / BQ) : 0;
+    // sliding window: the last row that sees a key of this workgroup
+    const int wg_rhi = CAUSAL ? min(a.M - 1, n0 + BK - 1 - a.gap + a.win - 1) : a.M - 1;
+    if (CAUSAL) nQtiles = min(nQtiles, max(0, wg_rhi + 1 + BQ - 1) / BQ);
     if (DOC) {
       ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
       eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
@@ -581,11 +586,15 @@ void bwd_dkdv_kernel(const KArgs a) {
       bool skip, lim, doc = false, glob = false, col = false;
       if (!DOC) {
         const int m0 = t * BQ;
-        skip = (nw >= a.N) || (CAUSAL && (a.gap + m0 + BQ - 1 < nw));
-        lim = (m0 + BQ > a.M) || (nw + 32 > a.N) || (CAUSAL && (a.gap + m0 < nw + 31));
+        const int rmin = m0, rmax = min(m0 + BQ - 1, a.M - 1);
+        skip = (nw >= a.N) || (CAUSAL && ((a.gap + rmax < nw && nw > a.pfx_m1) || a.gap + rmin - a.win + 1 > nw + 31));
+        lim = (m0 + BQ > a.M) || (nw + 32 > a.N) ||
+              (CAUSAL && ((a.gap + rmin < nw + 31 && nw + 31 > a.pfx_m1) || a.gap + rmax - a.win + 1 > nw));
       } else {
-        skip = (nw >= a.N) || (CAUSAL && (a.gap + qs.rmax < nw)) || !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
-        lim = (qs.nvalid < BQ) || (nw + 32 > a.N) || (CAUSAL && (a.gap + qs.rmin < nw + 31));
+        skip = (nw >= a.N) || (CAUSAL && ((a.gap + qs.rmax < nw && nw > a.pfx_m1) || a.gap + qs.rmin - a.win + 1 > nw + 31)) ||
+               !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
+        lim = (qs.nvalid < BQ) || (nw + 32 > a.N) ||
+              (CAUSAL && ((a.gap + qs.rmin < nw + 31 && nw + 31 > a.pfx_m1) || a.gap + qs.rmax - a.win + 1 > nw));
         doc = !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
         glob = qs.glob != 0;
         // one local id for the whole tile (padding rows aside, which the row-range mask drops):
@@ -596,7 +605,8 @@ void bwd_dkdv_kernel(const KArgs a) {
       return tile_value((skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0) | (col ? TF_COL : 0), qs.lo);
     };
     TileIter it;
-    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL ? n0 - a.gap : (int)0x80000000, dec);
+    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL && n0 > a.pfx_m1 ? n0 - a.gap : (int)0x80000000,
+                    CAUSAL ? wg_rhi : 0x7fffffff, dec);
     if (gi > 0) __syncthreads();  // the previous head's last tile may still be read from LDS
 
     // software pipeline: tile `cur` is computed while `nxt` streams into the other buffer and

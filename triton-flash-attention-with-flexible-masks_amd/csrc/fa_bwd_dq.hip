@@ -46,7 +46,7 @@ void bwd_dq_kernel(const KArgs a) {
   QTileCtx<CAUSAL, DOC> qc;
   if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
   q_work_finish(a, hd, wk);
-  int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
+  int kt_first = qc.first_tile(a), kt_last = qc.last_tile(a);
   const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
@@ -134,7 +134,7 @@ void bwd_dq_kernel(const KArgs a) {
       }
       if (need_lim) {
         asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
-        mask_lim(s, qc.lim_i - n0 - 32 * kb - 4 * g, 0.f);
+        mask_lim(s, qc.lim_i - n0 - 32 * kb - 4 * g, qc.low_i - n0 - 32 * kb - 4 * g, 0.f);
       }
       if (DOC && need_doc) {
         asm volatile("" ::: "memory");

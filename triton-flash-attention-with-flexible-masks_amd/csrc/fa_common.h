@@ -155,10 +155,12 @@ FA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 //   causal : gap + i >= j, gap = max(0, N - M)          flash_triton.py:107
 //   doc    : eq_i >= 0 || eq_i == ek_j                  flash_triton.py:114
 // ---------------------------------------------------------------------------
+//   window : j > gap + i - win (win = 0x3fffffff: off)    sliding window, causal only
+//   prefix : the causal term also holds for j <= pfx_m1   prefix-LM (pfx_m1 = -1: off)
 template <bool CAUSAL, bool DOC>
-FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j) {
+FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j, int win, int pfx_m1) {
   bool keep = j < N;
-  if (CAUSAL) keep = keep && (gap + i >= j);
+  if (CAUSAL) keep = keep && ((gap + i >= j) || (j <= pfx_m1)) && (j > gap + i - win);
   if (DOC) keep = keep && ((eq_i >= 0) || (eq_i == ek_j));
   return keep;
 }
@@ -236,6 +238,8 @@ struct KArgs {
   int64_t qs_bs, qs_hs;   // strides of qsum in entries
   int64_t ks_bs, ks_hs;
   int B, H, Hk, G, M, N, gap;
+  int win;      // sliding window: a row sees keys j > gap + i - win (0x3fffffff: no window)
+  int pfx_m1;   // prefix-LM: keys j <= pfx_m1 are seen by every row (-1: no prefix)
   int Pp;                 // entries of the permuted order per (b, h)
   int nQs, nKs;           // summary entries per (b, h)
   float scale;            // sm_scale

@@ -134,10 +134,12 @@ void fwd_f32_kernel(const KArgs a) {
   }
   const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
   const bool glob_i = eq_i >= 0;
-  const int lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;   // last key this row may see
+  const int lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;   // last key this row may see
+  const int low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;                 // first one (sliding window)
   // the wave's rows: largest such limit, id interval of the local rows, any global row
   const int w_last = min(mw + 31, a.M - 1);
-  const int w_lim = CAUSAL ? min(a.gap + w_last, a.N - 1) : a.N - 1;
+  const int w_lim = CAUSAL ? min(max(a.gap + w_last, a.pfx_m1), a.N - 1) : a.N - 1;
+  const int w_low = CAUSAL ? a.gap + mw - a.win + 1 : -0x3fffffff;   // smallest first key among the wave's rows
   int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
   if (DOC) {
     const bool live = row < a.M;
@@ -145,7 +147,8 @@ void fwd_f32_kernel(const KArgs a) {
     w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
     w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
   }
-  const int n_end = CAUSAL ? min(a.N, a.gap + min(m0 + 127, a.M - 1) + 1) : a.N;
+  const int n_end = CAUSAL ? min(a.N, max(a.gap + min(m0 + 127, a.M - 1), a.pfx_m1) + 1) : a.N;
+  const int kt0 = CAUSAL ? max(0, a.gap + m0 - a.win + 1) / kRows : 0;   // sliding window: first tile any row sees
   const int nkt = (n_end + kRows - 1) / kRows;   // the same for all waves: the tile stream has barriers
 
   f32x16 o[DBN];
@@ -157,11 +160,11 @@ void fwd_f32_kernel(const KArgs a) {
 
   TileRegs<D> rk, rv;
   int rid = 0;
-  rk.load(kp, a.k_rs, 0, a.N);
-  rv.load(vp, a.v_rs, 0, a.N);
-  if (DOC && threadIdx.x < kRows) rid = ekp[min((int)threadIdx.x, a.N - 1)];
+  rk.load(kp, a.k_rs, kt0 * kRows, a.N);
+  rv.load(vp, a.v_rs, kt0 * kRows, a.N);
+  if (DOC && threadIdx.x < kRows) rid = ekp[min(kt0 * kRows + (int)threadIdx.x, a.N - 1)];
 
-  for (int kt = 0; kt < nkt; ++kt) {
+  for (int kt = kt0; kt < nkt; ++kt) {
     const int n0 = kt * kRows;
     __syncthreads();   // the previous tile is no longer read
     rk.store(lk);
@@ -173,7 +176,7 @@ void fwd_f32_kernel(const KArgs a) {
       rv.load(vp, a.v_rs, n0 + kRows, a.N);
       if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
     }
-    bool skip = mw >= a.M || n0 > w_lim;
+    bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
       const int id = lid[lq];
@@ -187,7 +190,7 @@ void fwd_f32_kernel(const KArgs a) {
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
     pipelined<KS2, kChunk>([&](int i) __attribute__((always_inline)) { return lk[lq * RS + 2 * i + g]; },
                            [&](int i, float x) __attribute__((always_inline)) { s = mfma_f32(x, qreg[i], s); });
-    mask_lim(s, lim_i - n0 - 4 * g, -INFINITY);
+    mask_lim(s, lim_i - n0 - 4 * g, low_i - n0 - 4 * g, -INFINITY);
     if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, -INFINITY);
 
     float mx = s[0];
@@ -269,9 +272,11 @@ void dq_f32_kernel(const KArgs a) {
   const float delta_i = a.delta[(int64_t(b) * a.H + h) * a.M + rowc];
   const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
   const bool glob_i = eq_i >= 0;
-  const int lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;
+  const int lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;
+  const int low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;
   const int w_last = min(mw + 31, a.M - 1);
-  const int w_lim = CAUSAL ? min(a.gap + w_last, a.N - 1) : a.N - 1;
+  const int w_lim = CAUSAL ? min(max(a.gap + w_last, a.pfx_m1), a.N - 1) : a.N - 1;
+  const int w_low = CAUSAL ? a.gap + mw - a.win + 1 : -0x3fffffff;   // smallest first key among the wave's rows
   int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
   if (DOC) {
     const bool live = row < a.M;
@@ -279,7 +284,8 @@ void dq_f32_kernel(const KArgs a) {
     w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
     w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
   }
-  const int n_end = CAUSAL ? min(a.N, a.gap + min(m0 + 127, a.M - 1) + 1) : a.N;
+  const int n_end = CAUSAL ? min(a.N, max(a.gap + min(m0 + 127, a.M - 1), a.pfx_m1) + 1) : a.N;
+  const int kt0 = CAUSAL ? max(0, a.gap + m0 - a.win + 1) / kRows : 0;   // sliding window: first tile any row sees
   const int nkt = (n_end + kRows - 1) / kRows;
 
   f32x16 acc[DBN];
@@ -290,11 +296,11 @@ void dq_f32_kernel(const KArgs a) {
 
   TileRegs<D> rk, rv;
   int rid = 0;
-  rk.load(kp, a.k_rs, 0, a.N);
-  rv.load(vp, a.v_rs, 0, a.N);
-  if (DOC && threadIdx.x < kRows) rid = ekp[min((int)threadIdx.x, a.N - 1)];
+  rk.load(kp, a.k_rs, kt0 * kRows, a.N);
+  rv.load(vp, a.v_rs, kt0 * kRows, a.N);
+  if (DOC && threadIdx.x < kRows) rid = ekp[min(kt0 * kRows + (int)threadIdx.x, a.N - 1)];
 
-  for (int kt = 0; kt < nkt; ++kt) {
+  for (int kt = kt0; kt < nkt; ++kt) {
     const int n0 = kt * kRows;
     __syncthreads();
     rk.store(lk);
@@ -306,7 +312,7 @@ void dq_f32_kernel(const KArgs a) {
       rv.load(vp, a.v_rs, n0 + kRows, a.N);
       if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
     }
-    bool skip = mw >= a.M || n0 > w_lim;
+    bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
       const int id = lid[lq];
@@ -327,7 +333,7 @@ void dq_f32_kernel(const KArgs a) {
     // dS = P (dP - delta); masked pairs -> 0 (a select, so an overflowed exponential of a masked pair is harmless)
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = fast_exp2(__builtin_fmaf(s[r], c, -L_i)) * (dp[r] - delta_i);
-    mask_lim(s, lim_i - n0 - 4 * g, 0.f);
+    mask_lim(s, lim_i - n0 - 4 * g, low_i - n0 - 4 * g, 0.f);
     if (DOC) mask_doc(s, reinterpret_cast<const char*>(lid) + g * 16, eq_i, glob_i, 0.f);
     // dQ^T += K^T dS^T
     pipelined<16 * DBN, kChunk>(
@@ -379,10 +385,13 @@ void dkdv_f32_kernel(const KArgs a) {
   for (int s = 0; s < KS2; ++s) { kreg[s] = kp[2 * s + g]; vreg[s] = vp[2 * s + g]; }
   const float c = a.scale_log2e;
   // rows that may see this lane's key: [row_lo, row_lo + row_span)
-  const int row_lo = CAUSAL ? max(0, key - a.gap) : 0;
-  const unsigned row_span = key < a.N ? (unsigned)(a.M - row_lo) : 0u;
-  const int mt0 = CAUSAL ? max(0, n0 - a.gap) / kRows : 0;
-  const int nMt = (a.M + kRows - 1) / kRows;
+  // (causal: from the diagonal on, or from row 0 for a key of the prefix; sliding window: `win` rows)
+  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - a.gap)) : 0;
+  const int row_hi = CAUSAL ? min(a.M - 1, key - a.gap + a.win - 1) : a.M - 1;
+  const unsigned row_span = (key < a.N && row_hi >= row_lo) ? (unsigned)(row_hi - row_lo + 1) : 0u;
+  const int mt0 = CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - a.gap) / kRows) : 0;
+  const int wg_rhi = CAUSAL ? min(a.M - 1, n0 + 127 - a.gap + a.win - 1) : a.M - 1;   // last row that sees a key of the workgroup
+  const int nMt = max(0, wg_rhi + kRows) / kRows;
 
   f32x16 dv[DBN], dk[DBN];
 #pragma unroll
@@ -431,7 +440,8 @@ void dkdv_f32_kernel(const KArgs a) {
         rdo.load(dop, a.do_rs, m0 + kRows, a.M);
         if (threadIdx.x < 3 * kRows) raux = aux_load(m0 + kRows);
       }
-      bool skip = nw >= a.N || (CAUSAL && a.gap + min(m0 + kRows - 1, a.M - 1) < nw);
+      bool skip = nw >= a.N || (CAUSAL && ((a.gap + min(m0 + kRows - 1, a.M - 1) < nw && nw > a.pfx_m1) ||
+                                           a.gap + m0 - a.win + 1 > nw + 31));
       if (DOC && !skip) {
         const bool rv_ = m0 + lq < a.M;
         const int id = leq[lq];

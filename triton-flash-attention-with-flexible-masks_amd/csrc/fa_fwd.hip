@@ -58,7 +58,7 @@ void fwd_kernel(const KArgs a) {
   QTileCtx<CAUSAL, DOC> qc;
   if (!qc.init(a, b, h, wk.tile, threadIdx.x >> 6)) return;
   q_work_finish(a, hd, wk);
-  int kt_first = qc.first_tile(), kt_last = qc.last_tile(a);
+  int kt_first = qc.first_tile(a), kt_last = qc.last_tile(a);
   const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
@@ -149,8 +149,9 @@ void fwd_kernel(const KArgs a) {
     if (need_lim) {
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
       const int rel = qc.lim_i - n0 - 4 * g;
-      mask_lim(s[0], rel, -INFINITY);
-      mask_lim(s[1], rel - 32, -INFINITY);
+      const int rel_lo = qc.low_i - n0 - 4 * g;
+      mask_lim(s[0], rel, rel_lo, -INFINITY);
+      mask_lim(s[1], rel - 32, rel_lo - 32, -INFINITY);
     }
     if (DOC && need_doc) {
       asm volatile("" ::: "memory");

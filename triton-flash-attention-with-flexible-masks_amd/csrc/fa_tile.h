@@ -170,7 +170,8 @@ FA_DEV typename E::vec8 lds_tr8(const char* p0, const char* p1) {
 //                 [first, last) in natural order
 //   query mode  : own side = key tile (lo, hi), candidates = tiles of the permuted
 //                 query order; a tile is a candidate if it holds rows and, with a
-//                 causal mask, its largest row index reaches the own keys
+//                 causal mask, its largest row index reaches the own keys (and, with a sliding
+//                 window, its smallest row index is not past them)
 // With sum == nullptr (no document ids) every tile of the range is visited.
 // ---------------------------------------------------------------------------
 // Wave-level decisions for one tile, taken when the candidates are tested (dec(tile, summary) is
@@ -189,18 +190,19 @@ struct TileIter {
   int base, last;
   int flags;                  // TF_ bits of the tile returned by the last next()
   int o_lo, o_hi, o_glob;
-  int min_rmax;            // query mode: candidates need rmax >= min_rmax
+  int min_rmax, max_rmin;  // query mode: candidates need rmax >= min_rmax and rmin <= max_rmin
   bool keys_mode;
   const IdSummary* sum;
 
   template <class Dec>
   FA_DEV void init_keys(int first, int last_, const IdSummary* ksum, int q_lo, int q_hi, int q_glob, const Dec& dec) {
-    sum = ksum; o_lo = q_lo; o_hi = q_hi; o_glob = q_glob; keys_mode = true; min_rmax = 0;
+    sum = ksum; o_lo = q_lo; o_hi = q_hi; o_glob = q_glob; keys_mode = true; min_rmax = 0; max_rmin = 0x7fffffff;
     start(first, last_, dec);
   }
   template <class Dec>
-  FA_DEV void init_queries(int first, int last_, const IdSummary* qsum, int k_lo, int k_hi, int min_rmax_, const Dec& dec) {
-    sum = qsum; o_lo = k_lo; o_hi = k_hi; o_glob = 0; keys_mode = false; min_rmax = min_rmax_;
+  FA_DEV void init_queries(int first, int last_, const IdSummary* qsum, int k_lo, int k_hi, int min_rmax_, int max_rmin_,
+                           const Dec& dec) {
+    sum = qsum; o_lo = k_lo; o_hi = k_hi; o_glob = 0; keys_mode = false; min_rmax = min_rmax_; max_rmin = max_rmin_;
     start(first, last_, dec);
   }
   template <class Dec>
@@ -218,7 +220,7 @@ struct TileIter {
     if (sum != nullptr && v) {
       s = sum[t];
       v = keys_mode ? doc_may_keep(o_lo, o_hi, o_glob, s.lo, s.hi)
-                    : (s.nvalid > 0 && s.rmax >= min_rmax && doc_may_keep(s.lo, s.hi, s.glob, o_lo, o_hi));
+                    : (s.nvalid > 0 && s.rmax >= min_rmax && s.rmin <= max_rmin && doc_may_keep(s.lo, s.hi, s.glob, o_lo, o_hi));
     }
     const long long fv = dec(t, s);
     const int f = (int)fv;
@@ -256,10 +258,12 @@ struct QTileCtx {
   int rowc;   // row clamped into [0, M) for loads
   int eq_i;
   int w_lo, w_hi, w_glob, w_rmin, w_rmax;  // this wave's 32 rows
-  int g_lo, g_hi, g_glob, g_rmax;          // the workgroup's 128 rows
+  int g_lo, g_hi, g_glob, g_rmin, g_rmax;  // the workgroup's 128 rows
   int g_kfirst, g_klast;                   // key tiles (of 64) those rows can need, from the mask plan
-  int lim_i;                               // last key this lane's row may see (causal and length limit)
+  int lim_i;                               // last key this lane's row may see (causal / prefix and length limit)
   int w_limmin;                            // smallest such limit among the wave's rows
+  int low_i;                               // first key this lane's row may see (sliding window; very negative: none)
+  int w_lowmin, w_lowmax;                  // smallest / largest such bound among the wave's rows
   bool glob_i;                             // this lane's row has an id >= 0 (sees every id)
   const int* ekp;
   const IdSummary* ksum;
@@ -278,7 +282,7 @@ struct QTileCtx {
       row = mw + lq < a.M ? mw + lq : -1;
       w_rmin = mw; w_rmax = min(mw + 31, a.M - 1);
       if (w_rmax < w_rmin) w_rmax = -1;
-      g_rmax = min(m0 + 127, a.M - 1);
+      g_rmin = m0; g_rmax = min(m0 + 127, a.M - 1);
     } else {
       ekp = a.ek32 + b * a.ek_bs + h * a.ek_hs;
       ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
@@ -289,11 +293,11 @@ struct QTileCtx {
       eq_i = a.peq[pos];
       if (s0.nvalid + s1.nvalid == 0) {  // no rows: every decision below says "skip"
         row = -1; rowc = 0; eq_i = 0; w_rmin = 0x7fffffff; w_rmax = -1; w_glob = 0;
-        g_lo = 0x7fffffff; g_hi = (int)0x80000000; g_glob = 0; g_rmax = -1;
+        g_lo = 0x7fffffff; g_hi = (int)0x80000000; g_glob = 0; g_rmin = 0x7fffffff; g_rmax = -1;
         return false;
       }
       g_lo = min(s0.lo, s1.lo); g_hi = max(s0.hi, s1.hi); g_glob = s0.glob | s1.glob;
-      g_rmax = max(s0.rmax, s1.rmax);
+      g_rmin = min(s0.rmin, s1.rmin); g_rmax = max(s0.rmax, s1.rmax);
       g_kfirst = min(s0.kfirst, s1.kfirst); g_klast = max(s0.klast, s1.klast);
       const bool local = (eq_i < 0) && (row >= 0);
       int lo = local ? eq_i : 0x7fffffff, hi = local ? eq_i : (int)0x80000000;
@@ -309,15 +313,21 @@ struct QTileCtx {
       w_glob = __builtin_amdgcn_ballot_w64(eq_i >= 0 && row >= 0) != 0;
     }
     rowc = row >= 0 ? row : 0;
-    lim_i = CAUSAL ? min(a.gap + rowc, a.N - 1) : a.N - 1;
-    w_limmin = CAUSAL ? min(a.gap + w_rmin, a.N - 1) : a.N - 1;
+    lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;
+    w_limmin = CAUSAL ? min(max(a.gap + w_rmin, a.pfx_m1), a.N - 1) : a.N - 1;
+    low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;
+    w_lowmin = CAUSAL && w_rmax >= 0 ? a.gap + w_rmin - a.win + 1 : -0x3fffffff;
+    w_lowmax = CAUSAL && w_rmax >= 0 ? a.gap + w_rmax - a.win + 1 : -0x3fffffff;
     glob_i = eq_i >= 0;
     return true;
   }
   // range [first, last) of 64-key tiles the workgroup has to look at
-  FA_DEV int first_tile() const { return g_kfirst < 0x3fffffff ? g_kfirst : 0; }
+  FA_DEV int first_tile(const KArgs& a) const {
+    const int f = g_kfirst < 0x3fffffff ? g_kfirst : 0;
+    return CAUSAL && g_rmax >= 0 ? max(f, max(0, a.gap + g_rmin - a.win + 1) / 64) : f;   // sliding window
+  }
   FA_DEV int last_tile(const KArgs& a) const {
-    const int hi_key = CAUSAL ? min(a.N, a.gap + g_rmax + 1) : a.N;
+    const int hi_key = CAUSAL ? min(a.N, max(a.gap + g_rmax, a.pfx_m1) + 1) : a.N;
     return min((hi_key + 63) / 64, g_klast + 1);
   }
 
@@ -326,8 +336,8 @@ struct QTileCtx {
   //   TF_LIM  : some pair fails the causal / length limit  -> mask_lim
   //   TF_DOC  : some pair may fail the id test             -> mask_doc
   FA_DEV int decide(const KArgs& a, int n0, int BN, int k_lo, int k_hi) const {
-    bool skip = (w_rmax < 0) || (CAUSAL && (n0 > a.gap + w_rmax));
-    const bool need_lim = n0 + BN - 1 > w_limmin;
+    bool skip = (w_rmax < 0) || (CAUSAL && (n0 > max(a.gap + w_rmax, a.pfx_m1) || n0 + BN - 1 < w_lowmin));
+    const bool need_lim = n0 + BN - 1 > w_limmin || n0 < w_lowmax;
     bool need_doc = false;
     if (DOC) {
       skip = skip || !doc_may_keep(w_lo, w_hi, w_glob, k_lo, k_hi);
@@ -339,12 +349,17 @@ struct QTileCtx {
 
 // Element masks of one 32-key block held in the transposed-score layout: register 4*q4 + t of a
 // lane is key 8*q4 + 4*(lane >> 5) + t of the block.  Both are called under wave-uniform branches.
-//   rel  : (last key the lane's row may see) - (first key of the block) - 4*(lane >> 5)
-FA_DEV void mask_lim(f32x16& s, int rel, float fill) {
+//   rel    : (last key the lane's row may see) - (first key of the block) - 4*(lane >> 5)
+//   rel_lo : (first key the lane's row may see) - (first key of the block) - 4*(lane >> 5); both
+//            bounds in one unsigned compare (rel_lo is very negative without a sliding window)
+FA_DEV void mask_lim(f32x16& s, int rel, int rel_lo, float fill) {
+  const bool none = rel < rel_lo;   // empty interval: nothing may pass
+  const unsigned span = none ? 0u : (unsigned)(rel - rel_lo);
+  if (none) rel_lo = 0x3fffffff;
 #pragma unroll
   for (int q4 = 0; q4 < 4; ++q4)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (8 * q4 + t <= rel) ? s[4 * q4 + t] : fill;
+    for (int t = 0; t < 4; ++t) s[4 * q4 + t] = ((unsigned)(8 * q4 + t - rel_lo) <= span) ? s[4 * q4 + t] : fill;
 }
 //   ids  : LDS copy of the block's 32 key ids, already offset by 16*(lane >> 5) bytes
 // The four id vectors are requested together (one LDS round trip instead of four serial ones:

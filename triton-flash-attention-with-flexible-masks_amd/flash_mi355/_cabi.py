@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libflash_mi355.so"
 
-FA_ABI_VERSION = 1
+FA_ABI_VERSION = 2
 FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
 FA_DTYPE_BF16 = 0
@@ -40,7 +40,7 @@ class FaParams(Structure):
         ("eq_stride", c_int64 * 3), ("ek_stride", c_int64 * 3),
         ("B", c_int32), ("H", c_int32), ("Hk", c_int32), ("M", c_int32), ("N", c_int32), ("D", c_int32),
         ("causal", c_int32), ("score_mode", c_int32), ("dtype", c_int32), ("id_dtype", c_int32),
-        ("sm_scale", c_float), ("flags", c_int32),
+        ("sm_scale", c_float), ("flags", c_int32), ("window", c_int32), ("prefix", c_int32),
     ]
 
 

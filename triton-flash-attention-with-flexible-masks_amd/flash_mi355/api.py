@@ -50,7 +50,7 @@ def _stream_ptr(device) -> int:
 class _Plan:
     """fa_params filled in for one problem, plus the tensors that keep its pointers alive."""
 
-    def __init__(self, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+    def __init__(self, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
         B, H, M, D = q.shape
         N, Hk = k.shape[2], k.shape[1]
         p = _cabi.FaParams()
@@ -62,6 +62,7 @@ class _Plan:
         p.dtype = _DTYPES[q.dtype]
         p.sm_scale = float(sm_scale)
         p.flags = 0
+        p.window, p.prefix = int(window), int(prefix)
         self.keep = [q, k, v]
         if score_func_mode != SCORE_FUNC_MODE0_NOPE:
             p.eq, p.ek = eq.data_ptr(), ek.data_ptr()
@@ -109,7 +110,7 @@ class _Impl:
     """Forward and backward shared by the two autograd functions below."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
         # -- checks of flash_triton.py:510-530, same order and messages --
         Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
         assert Dq == Dk and Dk == Dv, "feature size of q, k, v should be equal"
@@ -130,6 +131,9 @@ class _Impl:
             assert score_func_mode == SCORE_FUNC_MODE0_NOPE
         # -- checks the reference leaves to the Triton launcher --
         assert score_func_mode in (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC), "unknown score_func_mode"
+        window, prefix = int(window or 0), int(prefix or 0)
+        assert window >= 0 and prefix >= 0 and not (window and prefix), "window and prefix exclude each other"
+        assert causal or not (window or prefix), "window / prefix are causal masks"
         assert q.is_cuda and k.is_cuda and v.is_cuda, "flash_mi355 runs on the GPU only"
         assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, \
             "q, k, v must share one of torch.bfloat16 / torch.float16 / torch.float32"
@@ -146,7 +150,7 @@ class _Impl:
 
         L = _cabi.lib()
         with torch.cuda.device(q.device):
-            plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+            plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
             Out = torch.empty_like(q)   # q's layout when q is dense (flash_triton.py:539), contiguous otherwise
             lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
             p = plan.p
@@ -158,18 +162,18 @@ class _Impl:
         ctx.sm_scale = sm_scale
         ctx.causal = causal
         ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
-        ctx.score_func_info = (score_func_mode,)
+        ctx.score_func_info = (score_func_mode, window, prefix)
         return Out, lse
 
     @staticmethod
     def backward(ctx, do, dlse):
         q, k, v, o, lse, eq, ek, workspace = ctx.saved_tensors
         B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
-        score_func_mode, = ctx.score_func_info
+        score_func_mode, window, prefix = ctx.score_func_info
         L = _cabi.lib()
         do = _aligned(maybe_contiguous(do))
         with torch.cuda.device(q.device):
-            plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode)
+            plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix)
             p = plan.p
             if workspace is not None:   # the forward's mask plan is reused as is
                 plan.restore(workspace, q.device)
@@ -190,7 +194,7 @@ class _Impl:
                 delta.sub_(torch.where(torch.isinf(lse), torch.zeros_like(lse), dlse.to(torch.float32)))
             _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
             _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
-        return dq, dk, dv, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 _forward, _backward = _Impl.forward, _Impl.backward
@@ -200,8 +204,8 @@ class FlashAttention(torch.autograd.Function):
     """Mirror of the reference autograd function (flash_triton.py:506-638)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
-        return _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)[0]
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
+        return _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)[0]
 
     @staticmethod
     def backward(ctx, do):
@@ -214,8 +218,8 @@ class FlashAttentionWithLse(torch.autograd.Function):
     entry point returns Out only, flash_triton.py:564)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode):
-        out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
+        out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
         return out, lse * math.log(2.0)
 
     @staticmethod
@@ -223,19 +227,22 @@ class FlashAttentionWithLse(torch.autograd.Function):
         return _backward(ctx, do, dlse)
 
 
-def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE):
-    """flash_triton.py:640-641."""
-    return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE,
+              *, window=0, prefix=0):
+    """flash_triton.py:640-641.  Two keyword-only additions, both causal masks (0 = off, exclusive):
+    window = W: sliding window, a row sees only its last W keys up to the diagonal;
+    prefix = P: prefix-LM, the first P keys are seen by every row."""
+    return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
 
 
 # ---------------------------------------------------------------------------
 # Accessors for tests and benchmarks (not part of the reference's surface).
 # ---------------------------------------------------------------------------
 def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
-                       score_func_mode=SCORE_FUNC_MODE0_NOPE):
+                       score_func_mode=SCORE_FUNC_MODE0_NOPE, *, window=0, prefix=0):
     """(O, LSE) with LSE in natural-log units (-inf for rows without a kept key); differentiable
     through both results."""
-    return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode)
+    return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
 
 
 def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
@@ -247,7 +254,7 @@ def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
     return (-(seq + 1)).to(torch.int32)
 
 
-def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_scale=None):
+def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_scale=None, *, window=0):
     """Packed variable-length batch (the calling convention of varlen flash-attention kernels):
     q [total_q, H, D], k and v [total_k, Hk, D], cu_seqlens_* int tensors [S+1] of cumulative
     sequence lengths starting at 0.  Token i of sequence s attends to the keys of sequence s
@@ -271,11 +278,11 @@ def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_
     ek = eq if (same and Tk == Tq) else varlen_ids(cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k, Tk)
     q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (q, k, v))
     out = attention(q4, k4, v4, causal, sm_scale, eq.view(1, 1, Tq).expand(1, H, Tq), ek.view(1, 1, Tk).expand(1, H, Tk),
-                    SCORE_FUNC_MODE1_DOC)
+                    SCORE_FUNC_MODE1_DOC, window=window)
     return out.squeeze(0).transpose(0, 1)
 
 
-def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda"):
+def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda", window=0, prefix=0):
     """keep(i, j) as a bool tensor [B, H, M, N], evaluated by the device mask routine."""
     L = _cabi.lib()
     device = torch.device(device)
@@ -283,6 +290,7 @@ def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_M
     p.B, p.H, p.Hk, p.M, p.N, p.D = B, H, H, M, N, 64
     p.causal = 1 if causal else 0
     p.score_mode = int(score_func_mode)
+    p.window, p.prefix = int(window), int(prefix)
     p.dtype = _cabi.FA_DTYPE_BF16
     keep = []
     with torch.cuda.device(device):
