@@ -519,3 +519,30 @@ def test_window_needs_causal():
         attention(q, q, q, False, window=8)
     with pytest.raises(AssertionError):
         attention(q, q, q, True, window=8, prefix=8)
+
+
+@pytest.mark.parametrize("seed", list(range(200, 232)))
+def test_random_shapes_all_types_and_masks(seed):
+    """Second seeded sweep: the three element types, and on causal draws a sliding window or a
+    prefix of random size (from a single key to longer than the sequence), with and without ids."""
+    rng = np.random.default_rng(seed)
+    D = int(rng.choice([16, 32, 64, 128]))
+    Hk = int(rng.choice([1, 2]))
+    H = Hk * int(rng.choice([1, 2, 3]))
+    B = int(rng.choice([1, 2]))
+    causal = bool(rng.integers(0, 3) > 0)
+    doc = bool(rng.integers(0, 2))
+    M = int(rng.integers(1, 700))
+    N = int(rng.integers(M, 900)) if (causal or doc or rng.integers(0, 2)) else int(rng.integers(1, 900))
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+    window = prefix = 0
+    if causal:
+        which = int(rng.integers(0, 3))
+        if which == 1:
+            window = int(rng.choice([1, 2, 31, 64, 65, 200, N, N + 50])) if rng.integers(0, 2) else int(rng.integers(1, N + 1))
+        elif which == 2:
+            prefix = int(rng.choice([1, 63, 64, 129, N, N + 7])) if rng.integers(0, 2) else int(rng.integers(1, N + 1))
+    kind = str(rng.choice(["uniform", "uniform", "alllocal", "allglobal"]))
+    f32 = dtype == torch.float32
+    _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed=seed, ids_kind=kind, window=window, prefix=prefix,
+              tol_o=TOL_F32 if f32 else TOL_O, tol_lse=TOL_F32 if f32 else TOL_LSE)
