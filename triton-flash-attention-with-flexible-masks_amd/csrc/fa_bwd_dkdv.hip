@@ -385,75 +385,73 @@ void bwd_dkdv_kernel(const KArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     };
     // Both roles run the same MFMA streams (the accumulators never cross a role branch):
-    //   x0 = first(0) | score: P0 -> LDS | x1 = first(1) | score: P1 -> LDS | gradient: dS0 | second(0) | gradient: dS1 | second(1)
-    // so the gradient wave's first product of block 1 and its second product of block 0 fall into
-    // the score wave's exponentials, and the score wave's second products into the gradient wave's waits.
+    //   first(0) | score: P0 -> LDS | first(1) | score: P1 -> LDS | gradient: dS0 | second(0) | gradient: dS1 | second(1)
+    // so the gradient wave's first product of block 1 falls into the score wave's exponentials and
+    // the score wave's second products into the gradient wave's waits.  (Running dV0 before exp1 in
+    // the score wave, or dS1 before dK0 in the gradient wave, measured the same or slightly worse.)
     const char* rows = role == 0 ? lqt : ldo;   // rows operand of the first product
     const char* trp = role == 0 ? ldo : lqt;    // transposed operand of the second product
     f32x16 x[2];
     vec8 yf[2][2];   // P (score wave) or dS (gradient wave) per block, rounded to the element type
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      // LSE of this lane's 16 query rows of the block (row 8*q4 + 4*g + t): requested ahead of the
-      // product so that its LDS round trip is hidden
-      f32x4 Lv[4];
+    f32x4 Lv[2][4];  // LSE of this lane's 16 query rows of a block (row 8*q4 + 4*g + t)
+    // requested ahead of the product so that the LDS round trip is hidden
+    auto lse_load = [&](const int qb) __attribute__((always_inline)) {
       if (role == 0) {
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) Lv[q4] = *reinterpret_cast<const f32x4*>(aux + (32 * qb + 8 * q4 + 4 * g) * 4);
+        for (int q4 = 0; q4 < 4; ++q4) Lv[qb][q4] = *reinterpret_cast<const f32x4*>(aux + (32 * qb + 8 * q4 + 4 * g) * 4);
       }
-      x[qb] = first_product(rows, qb);
-      if (role == 0) {
-        char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
-        // S -> P
+    };
+    auto score_part = [&](const int qb) __attribute__((always_inline)) {   // S -> P, published
+      if (role != 0) return;
+      char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
+      for (int q4 = 0; q4 < 4; ++q4) {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) x[qb][4 * q4 + t] = fast_exp2(__builtin_fmaf(x[qb][4 * q4 + t], c, -Lv[q4][t]));
-        }
-        mask_p(x[qb], qb, flags, tile_id, m0, aux);
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-#pragma unroll
-          for (int t = 0; t < 8; t += 2) {
-            const typename E::vec2 pr = E::cvt2(x[qb][8 * half + t], x[qb][8 * half + t + 1]);
-            yf[qb][half][t] = pr[0]; yf[qb][half][t + 1] = pr[1];
-          }
-          *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[qb][half];
-        }
-        lds_flag_store(smem + FLAG_OFF + (qb * NKB + kb) * 4, pair_seq);
+        for (int t = 0; t < 4; ++t) x[qb][4 * q4 + t] = fast_exp2(__builtin_fmaf(x[qb][4 * q4 + t], c, -Lv[qb][q4][t]));
       }
-    }
+      mask_p(x[qb], qb, flags, tile_id, m0, aux);
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      if (role == 1) {
-        const char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
-        // LDS round trips are long under load: delta is requested before the wait, both halves of
-        // P together after it
-        f32x4 dl[4];
+      for (int half = 0; half < 2; ++half) {
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) dl[q4] = *reinterpret_cast<const f32x4*>(aux + 256 + (32 * qb + 8 * q4 + 4 * g) * 4);
-        const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
-        for (int spin = 0; spin < kPairSpinMax && __builtin_amdgcn_readfirstlane(lds_flag_load(fl)) != pair_seq; ++spin) __builtin_amdgcn_s_sleep(1);
-        vec8 pr8[2];
+        for (int t = 0; t < 8; t += 2) {
+          const typename E::vec2 pr = E::cvt2(x[qb][8 * half + t], x[qb][8 * half + t + 1]);
+          yf[qb][half][t] = pr[0]; yf[qb][half][t + 1] = pr[1];
+        }
+        *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[qb][half];
+      }
+      lds_flag_store(smem + FLAG_OFF + (qb * NKB + kb) * 4, pair_seq);
+    };
+    auto grad_part = [&](const int qb) __attribute__((always_inline)) {    // dS = P * (dP - delta)
+      if (role != 1) return;
+      const char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
+      // LDS round trips are long under load: delta is requested before the wait, both halves of
+      // P together after it
+      f32x4 dl[4];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const vec8*>(pbuf + half * 1024);
-        // dS = P * (dP - delta), rounded for the second product
+      for (int q4 = 0; q4 < 4; ++q4) dl[q4] = *reinterpret_cast<const f32x4*>(aux + 256 + (32 * qb + 8 * q4 + 4 * g) * 4);
+      const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
+      for (int spin = 0; spin < kPairSpinMax && __builtin_amdgcn_readfirstlane(lds_flag_load(fl)) != pair_seq; ++spin) __builtin_amdgcn_s_sleep(1);
+      vec8 pr8[2];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const f32x8 pv = __builtin_convertvector(pr8[half], f32x8);
+      for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const vec8*>(pbuf + half * 1024);
 #pragma unroll
-          for (int q2 = 0; q2 < 2; ++q2) {
+      for (int half = 0; half < 2; ++half) {
+        const f32x8 pv = __builtin_convertvector(pr8[half], f32x8);
 #pragma unroll
-            for (int t = 0; t < 4; t += 2) {
-              const int e = 4 * q2 + t;
-              const typename E::vec2 pr = E::cvt2(pv[e] * (x[qb][8 * half + e] - dl[2 * half + q2][t]), pv[e + 1] * (x[qb][8 * half + e + 1] - dl[2 * half + q2][t + 1]));
-              yf[qb][half][e] = pr[0]; yf[qb][half][e + 1] = pr[1];
-            }
+        for (int q2 = 0; q2 < 2; ++q2) {
+#pragma unroll
+          for (int t = 0; t < 4; t += 2) {
+            const int e = 4 * q2 + t;
+            const typename E::vec2 pr = E::cvt2(pv[e] * (x[qb][8 * half + e] - dl[2 * half + q2][t]), pv[e + 1] * (x[qb][8 * half + e + 1] - dl[2 * half + q2][t + 1]));
+            yf[qb][half][e] = pr[0]; yf[qb][half][e + 1] = pr[1];
           }
         }
       }
-      second_product(trp, yf[qb], qb);
-    }
+    };
+    lse_load(0); x[0] = first_product(rows, 0); score_part(0);
+    lse_load(1); x[1] = first_product(rows, 1); score_part(1);
+    grad_part(0); second_product(trp, yf[0], 0);
+    grad_part(1); second_product(trp, yf[1], 1);
   };
 
   // One query tile, both roles in one wave: S and dP are accumulated alternately, P and dS stay in
