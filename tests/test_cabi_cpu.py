@@ -147,3 +147,34 @@ def test_drop_in_module_name():
     extra = {n: p for n, p in sig.parameters.items() if n not in pos}
     assert all(p.kind == p.KEYWORD_ONLY and p.default == 0 for p in extra.values())     # additions stay out of the way
     assert [sig.parameters[n].default for n in pos][3:] == [False, None, None, None, 0]
+
+
+def test_header_is_plain_c_and_matches_the_binding(tmp_path):
+    """include/flash_mi355.h compiles as C (no C++ or HIP types in the boundary), a C program linked
+    against the library sees the same struct size as the ctypes mirror, and validation works from C."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "flash_mi355.h"
+int main(void) {
+  fa_params p;
+  memset(&p, 0, sizeof p);
+  printf("%d %llu %llu %d %s\n", fa_version(), (unsigned long long)fa_params_size(), (unsigned long long)sizeof(fa_params),
+         fa_validate(&p, 0), fa_error_string(fa_validate(&p, 0)));
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    lib_dir = _cabi.LIB_PATH.parent
+    inc = Path(__file__).resolve().parent.parent / "include"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), "-o", str(exe), f"-L{lib_dir}",
+                    "-lflash_mi355", f"-Wl,-rpath,{lib_dir}"], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 4)
+    assert int(out[0]) == _cabi.FA_ABI_VERSION
+    assert int(out[1]) == int(out[2]) == ctypes.sizeof(_cabi.FaParams)
+    assert int(out[3]) == -2 and "head dimension" in out[4]      # D = 0 is the first thing a zeroed struct fails
