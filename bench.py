@@ -48,8 +48,8 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {
     # bytes per launch: FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (factors from a 1 GiB copy in the same runs)
     ("cfg4_doc_causal_16k", "fa_bwd_dkdv"): 816_500_000,
-    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_380_000_000,
-    ("cfg4_doc_causal_16k", "fa_fwd"): 1_250_000_000,
+    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_430_000_000,
+    ("cfg4_doc_causal_16k", "fa_fwd"): 1_270_000_000,
 }
 
 
