@@ -546,3 +546,12 @@ def test_random_shapes_all_types_and_masks(seed):
     f32 = dtype == torch.float32
     _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed=seed, ids_kind=kind, window=window, prefix=prefix,
               tol_o=TOL_F32 if f32 else TOL_O, tol_lse=TOL_F32 if f32 else TOL_LSE)
+
+
+@pytest.mark.parametrize("B,H,Hk", [(1, 1, 1), (3, 1, 1), (1, 5, 5), (1, 6, 3), (7, 1, 1), (3, 3, 1), (1, 12, 4), (5, 2, 2)])
+def test_head_counts_that_do_not_fill_the_xcds_evenly(B, H, Hk):
+    """Batch x head counts that are not multiples of 8 (the workgroup -> XCD map has three cases:
+    whole heads per XCD, a head shared by several XCDs, (slot, head) pairs dealt round-robin), with
+    enough query tiles per head that every case deals more than one round, with and without ids."""
+    _run_case(B, H, Hk, 450, 450, 64, torch.bfloat16, True, True, seed=B * 100 + H)
+    _run_case(B, H, Hk, 520, 840, 128, torch.float16, True, False, seed=B * 100 + H + 1)
