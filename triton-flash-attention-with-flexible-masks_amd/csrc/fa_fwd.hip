@@ -22,6 +22,9 @@
 
 #include "fa_tile.h"
 
+#ifndef FA_FWD_PRE
+#define FA_FWD_PRE 4
+#endif
 #ifndef FA_FWD_PRE2
 #define FA_FWD_PRE2 4
 #endif
@@ -136,7 +139,7 @@ void fwd_kernel(const KArgs a) {
     // Instruction order of this region: keep several K fragments in flight ahead of the MFMA that
     // consumes them (an LDS read takes about as long as three MFMAs).
     {
-      constexpr int NQK = 2 * KS, PRE = NQK < 4 ? NQK : 4;
+      constexpr int NQK = 2 * KS, PRE = NQK < FA_FWD_PRE ? NQK : FA_FWD_PRE;
       __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
       for (int i = 0; i < NQK - PRE; ++i) {
