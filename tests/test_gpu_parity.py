@@ -555,3 +555,27 @@ def test_head_counts_that_do_not_fill_the_xcds_evenly(B, H, Hk):
     enough query tiles per head that every case deals more than one round, with and without ids."""
     _run_case(B, H, Hk, 450, 450, 64, torch.bfloat16, True, True, seed=B * 100 + H)
     _run_case(B, H, Hk, 520, 840, 128, torch.float16, True, False, seed=B * 100 + H + 1)
+
+
+def test_varlen_with_sliding_window():
+    """Packed sequences with a sliding window: inside every sequence the window counts that
+    sequence's own positions (the packed row's causal offset is the same for query and key)."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    lens, W_ = [150, 9, 260, 64], 48
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    T, H, D = int(cu[-1]), 2, 128
+    g = torch.Generator().manual_seed(13)
+    q, k, v, do = (torch.randn(T, H, D, generator=g).to(torch.bfloat16) for _ in range(4))
+    print("varlen window", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cu.cuda(), causal=True, window=W_)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for s in range(len(lens)):
+        a, b = int(cu[s]), int(cu[s + 1])
+        sl = lambda t: t[a:b].transpose(0, 1)[None]
+        ro, _, rdq, rdk, rdv = O.attention_autograd(sl(q), sl(k), sl(v), sl(do), True, None, None, None, 0, window=W_)
+        for name, got, ref in (("o", out.detach(), ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+            err = (sl(got.float().cpu()) - ref).abs().max().item()
+            assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), f"sequence {s} {name} err {err}"
