@@ -40,7 +40,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "triton-flash-attention-with-flexible-masks_amd"))
 
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}   # MI355X dense MFMA peak
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}   # MI355X dense MFMA peaks
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
@@ -68,7 +68,7 @@ def parse_args():
 
 
 def make_inputs(w, torch):
-    dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[w.dtype]
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[w.dtype]
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(0)
     q = torch.randn(w.B, w.H, w.Lq, w.D, device=dev, generator=g).to(dt)
@@ -233,7 +233,7 @@ def main():
 
     value = tf(3.5 * f_fwd["tile"], ms_per_step)
     line = {
-        "metric": "attention fwd+bwd TFLOP/s (bf16, doc+causal mask, tile-effective FLOPs)",
+        "metric": f"attention fwd+bwd TFLOP/s ({w.dtype}, {'doc+' if w.doc else ''}{'causal' if w.causal else 'no'} mask, tile-effective FLOPs)",
         "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",

@@ -78,6 +78,8 @@ def make_workload(name: str, seed: int = 0) -> Workload:
         ek = np.broadcast_to(ek, (B, Lk)).copy()
         eq = np.stack([_globalise(rng, ek[b, -Lq:], 0.05) for b in range(B)])   # the last 4 docs
         return Workload(name, B, H, H, Lq, Lk, D, "fp16", True, True, eq, ek)
+    if name == "fp32_causal_4k":     # the fp32 kernels at a size that fills the chip
+        return Workload(name, 1, 32, 32, 4096, 4096, 128, "fp32", True, False)
     if name == "plain_causal_16k":   # no ids: the dense efficiency of the same kernels
         return Workload(name, 1, 32, 32, 16384, 16384, 128, "bf16", True, False)
     raise KeyError(name)
