@@ -88,7 +88,7 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
     from flash_mi355.api import _Plan, _set4, _stream_ptr
     L = _cabi.lib()
     dev = q.device
-    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else 0)
+    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else 0, w.window, w.prefix)
     p = plan.p
     o = torch.empty_like(q)
     lse = torch.empty(w.B, w.H, w.Lq, device=dev, dtype=torch.float32)
@@ -175,7 +175,7 @@ def main():
 
     def step():
         q.grad = k.grad = v.grad = None
-        out = attention(q, k, v, w.causal, scale, eq, ek, mode)
+        out = attention(q, k, v, w.causal, scale, eq, ek, mode, window=w.window, prefix=w.prefix)
         out.backward(do)
 
     if args.copy_probe:

@@ -27,6 +27,8 @@ class Workload:
     doc: bool
     eq: Optional[np.ndarray] = None   # [B, Lq] int32 (shared by all heads)
     ek: Optional[np.ndarray] = None   # [B, Lk] int32
+    window: int = 0       # sliding window (causal only; 0 = off)
+    prefix: int = 0       # prefix-LM (causal only; 0 = off)
 
 
 def _pack_docs(rng, L, draw_len):
@@ -78,6 +80,8 @@ def make_workload(name: str, seed: int = 0) -> Workload:
         ek = np.broadcast_to(ek, (B, Lk)).copy()
         eq = np.stack([_globalise(rng, ek[b, -Lq:], 0.05) for b in range(B)])   # the last 4 docs
         return Workload(name, B, H, H, Lq, Lk, D, "fp16", True, True, eq, ek)
+    if name == "window1k_causal_16k":   # sliding window of 1024 keys over 16K tokens
+        return Workload(name, 1, 32, 32, 16384, 16384, 128, "bf16", True, False, window=1024)
     if name == "fp32_causal_4k":     # the fp32 kernels at a size that fills the chip
         return Workload(name, 1, 32, 32, 4096, 4096, 128, "fp32", True, False)
     if name == "plain_causal_16k":   # no ids: the dense efficiency of the same kernels
@@ -94,7 +98,13 @@ def keep_rows(w: Workload, b: int, i0: int, i1: int) -> np.ndarray:
     j = np.arange(w.Lk, dtype=np.int64)[None, :]
     keep = np.ones((i1 - i0, w.Lk), dtype=bool)
     if w.causal:
-        keep &= (max(0, w.Lk - w.Lq) + i) >= j
+        gap = max(0, w.Lk - w.Lq)
+        c = (gap + i) >= j
+        if w.prefix:
+            c |= j < w.prefix
+        if w.window:
+            c &= j > gap + i - w.window
+        keep &= c
     if w.doc:
         e_q = w.eq[b, i0:i1].astype(np.int64)[:, None]
         e_k = w.ek[b].astype(np.int64)[None, :]
@@ -173,6 +183,8 @@ def executed_wave_steps(w: Workload):
     32 keys.  Both cover 2048 score elements, i.e. 2048 * 4 * D FLOPs in the forward.
     """
     gap = max(0, w.Lk - w.Lq)
+    win = w.window if w.window else 2**30
+    pfx_m1 = min(w.prefix, w.Lk) - 1 if w.prefix else -1
     fwd_steps = kv_steps = 0
     nK64 = (w.Lk + 63) // 64
     nK32 = (w.Lk + 31) // 32
@@ -202,7 +214,7 @@ def executed_wave_steps(w: Workload):
         j0 = np.arange(nK64)[None, :] * 64
         vis = np.broadcast_to(nv[:, None] > 0, (len(nv), nK64)).copy()
         if w.causal:
-            vis = vis & (j0 <= gap + rmax[:, None])
+            vis = vis & (j0 <= np.maximum(gap + rmax[:, None], pfx_m1)) & (j0 + 63 >= gap + rmin[:, None] - win + 1)
         if w.doc:
             vis = vis & (g[:, None] | ((lo[:, None] <= k64_hi[None, :]) & (k64_lo[None, :] <= hi[:, None])))
         fwd_steps += int(vis.sum())
@@ -216,7 +228,7 @@ def executed_wave_steps(w: Workload):
         n0 = np.arange(nK32)[None, :] * 32
         vis = np.broadcast_to(nv[:, None] > 0, (len(nv), nK32)).copy()
         if w.causal:
-            vis = vis & (gap + rmax[:, None] >= n0)
+            vis = vis & ((gap + rmax[:, None] >= n0) | (n0 <= pfx_m1)) & (gap + rmin[:, None] - win + 1 <= n0 + 31)
         if w.doc:
             vis = vis & (g[:, None] | ((lo[:, None] <= k32_hi[None, :]) & (k32_lo[None, :] <= hi[:, None])))
         kv_steps += int(vis.sum())
