@@ -101,6 +101,8 @@ CASES = [
     (1, 2, 2, 256, 256, 16, torch.bfloat16, True, True),
     (2, 2, 1, 100, 300, 16, torch.float16, True, True),
     (1, 2, 2, 192, 192, 64, torch.bfloat16, False, False),
+    (1, 1, 1, 2048, 2048, 128, torch.bfloat16, False, False),  # long tile stream: the 128-key dk/dv form without ids
+    (1, 2, 1, 2100, 4300, 128, torch.float16, True, False),    # the same under a causal mask, grouped and ragged
 ]
 
 

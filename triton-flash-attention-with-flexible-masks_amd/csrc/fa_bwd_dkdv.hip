@@ -662,14 +662,12 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
 }
 
-template <typename Tag, int D, bool CAUSAL, bool DOC>
-static int launch_one(const KArgs& a, hipStream_t s) {
+#ifndef FA_KV_SHORT_TILES
+#define FA_KV_SHORT_TILES 32
+#endif
+template <typename Tag, int D, bool CAUSAL, bool DOC, int NKB>
+static int launch_nkb(const KArgs& a, hipStream_t s) {
   constexpr bool SPLIT = D > 64;
-  // With ids a workgroup visits few query tiles (a dozen at 16K tokens in documents of ~512), so its
-  // set-up and drain are a sizeable part of its life: two 64-key workgroups per CU cover each other's
-  // there (measured 9 % faster); without ids the tile stream is long and the 128-key form reads
-  // every query tile half as often (the 64-key form is 5 % slower there).
-  constexpr int NKB = SPLIT && DOC ? 2 : 4;
   constexpr int BK = 32 * NKB, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
   const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 + 64 : 0);
@@ -678,6 +676,25 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
   hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(SPLIT ? 128 * NKB : 64 * NKB), lds, s, a);
   return (int)hipGetLastError();
+}
+
+template <typename Tag, int D, bool CAUSAL, bool DOC>
+static int launch_one(const KArgs& a, hipStream_t s) {
+  // Role-split form (D = 128): a workgroup that visits few query tiles spends a sizeable part of its
+  // life in set-up and drain, and two 64-key workgroups per CU cover each other's there; a long tile
+  // stream is better served by the 128-key form, which reads every query tile half as often.  With
+  // ids a workgroup visits about a dozen tiles at 16K tokens in documents of ~512 (64-key form 9 %
+  // faster); without ids the number of tiles is known here: all of them, half on average under a
+  // causal mask, at most a window's worth under a sliding window.
+  if constexpr (D > 64) {
+    if (DOC) return launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s);
+    int tiles = (a.M + 63) / 64;
+    if (CAUSAL) tiles = a.win < 0x3fffffff ? min(tiles, a.win / 64 + 3) : (tiles + 1) / 2;
+    tiles *= a.G;
+    return tiles < FA_KV_SHORT_TILES ? launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s) : launch_nkb<Tag, D, CAUSAL, DOC, 4>(a, s);
+  } else {
+    return launch_nkb<Tag, D, CAUSAL, DOC, 4>(a, s);
+  }
 }
 
 template <typename Tag, int D>
