@@ -161,38 +161,59 @@ void fwd_kernel(const KArgs a) {
       mask_doc(s[0], lid, eq_i, qc.glob_i, -INFINITY);
       mask_doc(s[1], lid + 32 * 4, eq_i, qc.glob_i, -INFINITY);
     }
-    // online softmax in the exp2 domain with a lazily moved reference point
-    float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
-    float mx1 = fmaxf(fmaxf(s[1][0], s[1][1]), s[1][2]);
-#pragma unroll
-    for (int r = 3; r < 15; r += 2) {
-      mx0 = fmaxf(fmaxf(mx0, s[0][r]), s[0][r + 1]);
-      mx1 = fmaxf(fmaxf(mx1, s[1][r]), s[1][r + 1]);
-    }
-    float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(s[0][15], s[1][15]));
-    mx = xhalf_max(mx) * c;   // -inf stays -inf (c > 0)
-    if (__builtin_amdgcn_ballot_w64(mx - m_ref > RESCALE_THRESH) != 0) {
-      const float m_new = fmaxf(m_ref, mx);
-      // m_ref = -inf: nothing accumulated yet, alpha = exp2(-inf) = 0 (or NaN-free 0 below)
-      const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(m_ref - m_new);
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int db = 0; db < DBN; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
-    }
-    const float msub = (m_ref == -INFINITY) ? 0.f : m_ref;  // all scores -inf so far: exp2(-inf - 0) = 0
+    // Online softmax in the exp2 domain with a lazily moved reference point.  Fast path: the
+    // exponentials are taken against the reference point as it stands and only their sum is looked
+    // at -- while every lane's partial row sum stays below a limit no element can be large, so the
+    // row maximum (24 max operations, a lane exchange, the comparison) is not needed at all.  A
+    // reference point that is not set yet (-inf: the sum comes out inf or NaN) or too low sends the
+    // whole wave through the full path: row maximum, new reference point, O and l rescaled.
+    constexpr float kSumLimit = 4096.f;   // per lane over its 32 keys: every p <= 4096 (fits fp16 too)
+    f32x16 p[2];
     float ps0 = 0.f, ps1 = 0.f;
+    bool slow = __builtin_amdgcn_ballot_w64(m_ref == -INFINITY) != 0;
+    if (!slow) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float p0 = fast_exp2(__builtin_fmaf(s[0][r], c, -msub));
-      const float p1 = fast_exp2(__builtin_fmaf(s[1][r], c, -msub));
-      s[0][r] = p0;
-      s[1][r] = p1;
-      ps0 += p0;
-      ps1 += p1;
+      for (int r = 0; r < 16; ++r) {
+        p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -m_ref));
+        p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -m_ref));
+        ps0 += p[0][r];
+        ps1 += p[1][r];
+      }
+      slow = __builtin_amdgcn_ballot_w64(!(ps0 + ps1 <= kSumLimit)) != 0;
     }
+    if (slow) {
+      float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
+      float mx1 = fmaxf(fmaxf(s[1][0], s[1][1]), s[1][2]);
+#pragma unroll
+      for (int r = 3; r < 15; r += 2) {
+        mx0 = fmaxf(fmaxf(mx0, s[0][r]), s[0][r + 1]);
+        mx1 = fmaxf(fmaxf(mx1, s[1][r]), s[1][r + 1]);
+      }
+      float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(s[0][15], s[1][15]));
+      mx = xhalf_max(mx) * c;   // -inf stays -inf (c > 0)
+      if (__builtin_amdgcn_ballot_w64(mx - m_ref > RESCALE_THRESH) != 0) {
+        const float m_new = fmaxf(m_ref, mx);
+        // m_ref = -inf: nothing accumulated yet, alpha = exp2(-inf) = 0 (or NaN-free 0 below)
+        const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(m_ref - m_new);
+        m_ref = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < DBN; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      }
+      const float msub = (m_ref == -INFINITY) ? 0.f : m_ref;  // all scores -inf so far: exp2(-inf - 0) = 0
+      ps0 = 0.f; ps1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -msub));
+        p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -msub));
+        ps0 += p[0][r];
+        ps1 += p[1][r];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[0][r] = p[0][r]; s[1][r] = p[1][r]; }
     l_run += ps0 + ps1;
     // O^T += V^T P^T, 16 keys per MFMA.  V^T fragments (two transposed reads each) are requested
     // PRE MFMAs ahead in program order, P is converted just in time; the scheduling barriers pin
