@@ -41,7 +41,6 @@ void fwd_kernel(const KArgs a) {
   constexpr int DL = D < 32 ? 32 : D;  // LDS row width: D = 16 is staged as 32 columns, the upper 16 zero
   constexpr int DBN = DL / 32;
   constexpr int TILE_BYTES = BN * DL * 2;
-  constexpr float RESCALE_THRESH = 8.0f;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -106,7 +105,10 @@ void fwd_kernel(const KArgs a) {
   for (int db = 0; db < DBN; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
-  float m_ref = -INFINITY;  // scaled reference point of the exponentials (shared by lanes l, l^32)
+  // scaled reference point of the exponentials (shared by lanes l, l^32); "not set yet" is a huge
+  // negative finite number, so that exp2(s - m_ref) is 0 for a masked score and +inf for any other
+  constexpr float kUnset = -1e30f;
+  float m_ref = kUnset;
   float l_run = 0.f;        // this lane's partial row sum
 
   // One K/V tile; BUF is a compile-time constant so every LDS address is base + immediate.
@@ -165,23 +167,20 @@ void fwd_kernel(const KArgs a) {
     // exponentials are taken against the reference point as it stands and only their sum is looked
     // at -- while every lane's partial row sum stays below a limit no element can be large, so the
     // row maximum (24 max operations, a lane exchange, the comparison) is not needed at all.  A
-    // reference point that is not set yet (-inf: the sum comes out inf or NaN) or too low sends the
-    // whole wave through the full path: row maximum, new reference point, O and l rescaled.
+    // reference point that is not set yet (the sum comes out +inf) or too low sends the
+    // whole wave through the full path: row maximum, new reference point, O and l rescaled.  A row
+    // that has not met a kept key yet stays on the fast path (its exponentials are exact zeros).
     constexpr float kSumLimit = 4096.f;   // per lane over its 32 keys: every p <= 4096 (fits fp16 too)
     f32x16 p[2];
     float ps0 = 0.f, ps1 = 0.f;
-    bool slow = __builtin_amdgcn_ballot_w64(m_ref == -INFINITY) != 0;
-    if (!slow) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -m_ref));
-        p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -m_ref));
-        ps0 += p[0][r];
-        ps1 += p[1][r];
-      }
-      slow = __builtin_amdgcn_ballot_w64(!(ps0 + ps1 <= kSumLimit)) != 0;
+    for (int r = 0; r < 16; ++r) {
+      p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -m_ref));
+      p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -m_ref));
+      ps0 += p[0][r];
+      ps1 += p[1][r];
     }
-    if (slow) {
+    if (__builtin_amdgcn_ballot_w64(!(ps0 + ps1 <= kSumLimit)) != 0) {
       float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
       float mx1 = fmaxf(fmaxf(s[1][0], s[1][1]), s[1][2]);
 #pragma unroll
@@ -191,10 +190,11 @@ void fwd_kernel(const KArgs a) {
       }
       float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(s[0][15], s[1][15]));
       mx = xhalf_max(mx) * c;   // -inf stays -inf (c > 0)
-      if (__builtin_amdgcn_ballot_w64(mx - m_ref > RESCALE_THRESH) != 0) {
+      {
+        // the reference point moves to the running maximum whenever this path is taken (after it
+        // every p of the row is <= 1 again, so the next tiles are back on the fast path)
         const float m_new = fmaxf(m_ref, mx);
-        // m_ref = -inf: nothing accumulated yet, alpha = exp2(-inf) = 0 (or NaN-free 0 below)
-        const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(m_ref - m_new);
+        const float alpha = fast_exp2(m_ref - m_new);   // 0 when the reference point is set for the first time
         m_ref = m_new;
         l_run *= alpha;
 #pragma unroll
@@ -202,7 +202,7 @@ void fwd_kernel(const KArgs a) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
       }
-      const float msub = (m_ref == -INFINITY) ? 0.f : m_ref;  // all scores -inf so far: exp2(-inf - 0) = 0
+      const float msub = m_ref;   // still unset: every score of the row so far is -inf, exp2(-inf) = 0
       ps0 = 0.f; ps1 = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
