@@ -113,6 +113,7 @@ static KArgs make_args(const fa_params* p) {
   a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.pm_bs = a.pm_hs = a.qh_bs = a.qh_hs = 0;
   a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
   a.nQs = a.nKs = a.Pp = 0;
+  a.qk_same = 0;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     const WsLayout w = ws_layout(p);
     char* ws = reinterpret_cast<char*>(p->workspace);
@@ -130,6 +131,8 @@ static KArgs make_args(const fa_params* p) {
     a.qs_bs = int64_t(w.Hq1) * w.nQs; a.qs_hs = w.Hq1 == 1 ? 0 : w.nQs;
     a.ks_bs = int64_t(w.Hk1) * w.nKs; a.ks_hs = w.Hk1 == 1 ? 0 : w.nKs;
     a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
+    a.qk_same = (p->eq == p->ek && p->M == p->N && p->eq_stride[0] == p->ek_stride[0] && p->eq_stride[1] == p->ek_stride[1] &&
+                 p->eq_stride[2] == p->ek_stride[2]) ? 1 : 0;
     const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
     a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);

@@ -96,6 +96,18 @@ FA_DEV void pipelined(RD&& rd, MM&& mm) {
 }
 constexpr int kChunk = 8;
 
+// (min, max, or) of one value triple per wave over the 4 waves of the workgroup
+FA_DEV void wg_reduce3(int& lo, int& hi, int& glob) {
+  __shared__ int red[12];
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();   // a previous use of the buffer is over
+  if ((threadIdx.x & 63) == 0) { red[wave * 3] = lo; red[wave * 3 + 1] = hi; red[wave * 3 + 2] = glob; }
+  __syncthreads();
+  lo = min(min(red[0], red[3]), min(red[6], red[9]));
+  hi = max(max(red[1], red[4]), max(red[7], red[10]));
+  glob = red[2] | red[5] | red[8] | red[11];
+}
+
 template <int D>
 constexpr size_t lds_bytes() { return size_t(2 * kRows * (D + 1) + 4 * kRows + 64) * 4; }
 
@@ -160,22 +172,44 @@ void fwd_f32_kernel(const KArgs a) {
 
   TileRegs<D> rk, rv;
   int rid = 0;
-  rk.load(kp, a.k_rs, kt0 * kRows, a.N);
-  rv.load(vp, a.v_rs, kt0 * kRows, a.N);
-  if (DOC && threadIdx.x < kRows) rid = ekp[min(kt0 * kRows + (int)threadIdx.x, a.N - 1)];
+  // With ids, key tiles that no row of the workgroup can see (by the 64-key summaries of the mask
+  // plan) are not even loaded: a packed batch costs its block diagonal, not the whole triangle.
+  int g_lo = w_lo, g_hi = w_hi, g_glob = w_glob;
+  const IdSummary* ksum = nullptr;
+  if (DOC) {
+    wg_reduce3(g_lo, g_hi, g_glob);
+    ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
+  }
+  auto next_kt = [&](int kt) {
+    if (DOC)
+      while (kt < nkt) {
+        const IdSummary ks = ksum[(kt * kRows) / kSumRows];
+        if (doc_may_keep(g_lo, g_hi, g_glob, ks.lo, ks.hi)) break;
+        ++kt;
+      }
+    return kt;
+  };
+  int kt = next_kt(kt0);
+  if (kt < nkt) {
+    rk.load(kp, a.k_rs, kt * kRows, a.N);
+    rv.load(vp, a.v_rs, kt * kRows, a.N);
+    if (DOC && threadIdx.x < kRows) rid = ekp[min(kt * kRows + (int)threadIdx.x, a.N - 1)];
+  }
 
-  for (int kt = kt0; kt < nkt; ++kt) {
+  while (kt < nkt) {
     const int n0 = kt * kRows;
+    const int kt_next = next_kt(kt + 1);
     __syncthreads();   // the previous tile is no longer read
     rk.store(lk);
     rv.store(lv);
     if (DOC && threadIdx.x < kRows) lid[threadIdx.x] = rid;
     __syncthreads();
-    if (kt + 1 < nkt) {   // the next tile travels while this one is used
-      rk.load(kp, a.k_rs, n0 + kRows, a.N);
-      rv.load(vp, a.v_rs, n0 + kRows, a.N);
-      if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
+    if (kt_next < nkt) {   // the next tile travels while this one is used
+      rk.load(kp, a.k_rs, kt_next * kRows, a.N);
+      rv.load(vp, a.v_rs, kt_next * kRows, a.N);
+      if (DOC && threadIdx.x < kRows) rid = ekp[min(kt_next * kRows + (int)threadIdx.x, a.N - 1)];
     }
+    kt = kt_next;
     bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
@@ -296,22 +330,44 @@ void dq_f32_kernel(const KArgs a) {
 
   TileRegs<D> rk, rv;
   int rid = 0;
-  rk.load(kp, a.k_rs, kt0 * kRows, a.N);
-  rv.load(vp, a.v_rs, kt0 * kRows, a.N);
-  if (DOC && threadIdx.x < kRows) rid = ekp[min(kt0 * kRows + (int)threadIdx.x, a.N - 1)];
+  // With ids, key tiles that no row of the workgroup can see (by the 64-key summaries of the mask
+  // plan) are not even loaded: a packed batch costs its block diagonal, not the whole triangle.
+  int g_lo = w_lo, g_hi = w_hi, g_glob = w_glob;
+  const IdSummary* ksum = nullptr;
+  if (DOC) {
+    wg_reduce3(g_lo, g_hi, g_glob);
+    ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
+  }
+  auto next_kt = [&](int kt) {
+    if (DOC)
+      while (kt < nkt) {
+        const IdSummary ks = ksum[(kt * kRows) / kSumRows];
+        if (doc_may_keep(g_lo, g_hi, g_glob, ks.lo, ks.hi)) break;
+        ++kt;
+      }
+    return kt;
+  };
+  int kt = next_kt(kt0);
+  if (kt < nkt) {
+    rk.load(kp, a.k_rs, kt * kRows, a.N);
+    rv.load(vp, a.v_rs, kt * kRows, a.N);
+    if (DOC && threadIdx.x < kRows) rid = ekp[min(kt * kRows + (int)threadIdx.x, a.N - 1)];
+  }
 
-  for (int kt = kt0; kt < nkt; ++kt) {
+  while (kt < nkt) {
     const int n0 = kt * kRows;
+    const int kt_next = next_kt(kt + 1);
     __syncthreads();
     rk.store(lk);
     rv.store(lv);
     if (DOC && threadIdx.x < kRows) lid[threadIdx.x] = rid;
     __syncthreads();
-    if (kt + 1 < nkt) {
-      rk.load(kp, a.k_rs, n0 + kRows, a.N);
-      rv.load(vp, a.v_rs, n0 + kRows, a.N);
-      if (DOC && threadIdx.x < kRows) rid = ekp[min(n0 + kRows + (int)threadIdx.x, a.N - 1)];
+    if (kt_next < nkt) {
+      rk.load(kp, a.k_rs, kt_next * kRows, a.N);
+      rv.load(vp, a.v_rs, kt_next * kRows, a.N);
+      if (DOC && threadIdx.x < kRows) rid = ekp[min(kt_next * kRows + (int)threadIdx.x, a.N - 1)];
     }
+    kt = kt_next;
     bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
@@ -421,25 +477,45 @@ void dkdv_f32_kernel(const KArgs a) {
       if (which == 2 && DOC) return __int_as_float(eqp[r]);
       return 0.f;
     };
+    // When eq and ek are one id vector (self-attention), the 64-key summaries of the plan describe
+    // the query rows as well: query tiles that no key of the workgroup can meet are not even loaded.
+    int gk_lo = wk_lo, gk_hi = wk_hi, gk_unused = 0;
+    const IdSummary* rsum = nullptr;
+    if (DOC && a.qk_same) {
+      wg_reduce3(gk_lo, gk_hi, gk_unused);
+      rsum = a.ksum + b * a.ks_bs + h * a.ks_hs;
+    }
+    auto next_mt = [&](int mt) {
+      if (DOC && rsum != nullptr)
+        while (mt < nMt) {
+          const IdSummary qs = rsum[(mt * kRows) / kSumRows];   // ids of 64 rows: any id >= 0 is a global row
+          if (doc_may_keep(qs.lo, qs.hi, qs.hi >= 0, gk_lo, gk_hi)) break;
+          ++mt;
+        }
+      return mt;
+    };
     TileRegs<D> rq, rdo;
     float raux = 0.f;
-    if (mt0 < nMt) {
-      rq.load(qp, a.q_rs, mt0 * kRows, a.M);
-      rdo.load(dop, a.do_rs, mt0 * kRows, a.M);
-      if (threadIdx.x < 3 * kRows) raux = aux_load(mt0 * kRows);
+    int mt = next_mt(mt0);
+    if (mt < nMt) {
+      rq.load(qp, a.q_rs, mt * kRows, a.M);
+      rdo.load(dop, a.do_rs, mt * kRows, a.M);
+      if (threadIdx.x < 3 * kRows) raux = aux_load(mt * kRows);
     }
-    for (int mt = mt0; mt < nMt; ++mt) {
+    while (mt < nMt) {
       const int m0 = mt * kRows;
+      const int mt_next = next_mt(mt + 1);
       __syncthreads();
       rq.store(lqt);
       rdo.store(ldo);
       if (threadIdx.x < 3 * kRows) laux[threadIdx.x] = raux;
       __syncthreads();
-      if (mt + 1 < nMt) {
-        rq.load(qp, a.q_rs, m0 + kRows, a.M);
-        rdo.load(dop, a.do_rs, m0 + kRows, a.M);
-        if (threadIdx.x < 3 * kRows) raux = aux_load(m0 + kRows);
+      if (mt_next < nMt) {
+        rq.load(qp, a.q_rs, mt_next * kRows, a.M);
+        rdo.load(dop, a.do_rs, mt_next * kRows, a.M);
+        if (threadIdx.x < 3 * kRows) raux = aux_load(mt_next * kRows);
       }
+      mt = mt_next;
       bool skip = nw >= a.N || (CAUSAL && ((a.gap + min(m0 + kRows - 1, a.M - 1) < nw && nw > a.pfx_m1) ||
                                            a.gap + m0 - a.win + 1 > nw + 31));
       if (DOC && !skip) {
