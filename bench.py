@@ -48,8 +48,8 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {
     # bytes per launch: FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (factors from a 1 GiB copy in the same runs)
     ("cfg4_doc_causal_16k", "fa_bwd_dkdv"): 816_500_000,
-    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_430_000_000,
-    ("cfg4_doc_causal_16k", "fa_fwd"): 1_270_000_000,
+    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_562_000_000,
+    ("cfg4_doc_causal_16k", "fa_fwd"): 1_254_000_000,
 }
 
 
@@ -104,7 +104,13 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
     stream = _stream_ptr(dev)
     ref = ctypes.byref(p)
     out = {}
-    names = [("fa_fwd", L.fa_fwd), ("fa_bwd_delta", L.fa_bwd_delta), ("fa_bwd_dkdv", L.fa_bwd_dkdv), ("fa_bwd_dq", L.fa_bwd_dq)]
+    # the launches of the operator's backward: dq forms delta itself for the 16-bit types (as api.py asks
+    # for), fp32 keeps the separate delta launch
+    if w.dtype == "fp32":
+        names = [("fa_fwd", L.fa_fwd), ("fa_bwd_delta", L.fa_bwd_delta), ("fa_bwd_dkdv", L.fa_bwd_dkdv), ("fa_bwd_dq", L.fa_bwd_dq)]
+    else:
+        p.flags = _cabi.FA_FLAG_DQ_DELTA
+        names = [("fa_fwd", L.fa_fwd), ("fa_bwd_dq", L.fa_bwd_dq), ("fa_bwd_dkdv", L.fa_bwd_dkdv)]
     if w.doc:
         names.insert(0, ("fa_mask_plan", L.fa_mask_plan))
     for name, fn in names:
@@ -198,7 +204,7 @@ def main():
     f_fwd = W.flops(w, "fwd", kept, tiles)
     kt = time_kernels(w, q.detach(), k.detach(), v.detach(), do, eq, ek, torch)
     t_fwd = kt["fa_fwd"] + kt.get("fa_mask_plan", 0.0)
-    t_bwd = kt["fa_bwd_delta"] + kt["fa_bwd_dkdv"] + kt["fa_bwd_dq"]
+    t_bwd = kt.get("fa_bwd_delta", 0.0) + kt["fa_bwd_dkdv"] + kt["fa_bwd_dq"]
     peak = PEAK_TFLOPS[w.dtype]
 
     def tf(flops, ms):

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 2
+#define FA_ABI_VERSION 3
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
@@ -71,6 +71,12 @@ extern "C" {
 #define FA_ERR_WORKSPACE        -8   /* workspace missing or too small */
 #define FA_ERR_HIP              -9   /* kernel launch failed; see fa_last_hip_error */
 #define FA_ERR_NOT_IMPLEMENTED -10
+
+/* fa_params.flags */
+#define FA_FLAG_DQ_DELTA 1  /* fa_bwd_dq computes delta = rowsum(o * dout) of its own rows itself (o must be set)
+                               and also stores it to p->delta: the fa_bwd_delta launch is then not needed, and
+                               fa_bwd_dkdv, which reads delta, goes after fa_bwd_dq on the stream.
+                               16-bit dtypes only (FA_ERR_NOT_IMPLEMENTED for fp32).  Ignored by every other call. */
 
 typedef struct fa_params {
   /* forward operands */
@@ -103,7 +109,7 @@ typedef struct fa_params {
   int32_t dtype;          /* FA_DTYPE_*  (q,k,v,o,dout,dq,dk,dv share it) */
   int32_t id_dtype;       /* FA_IDTYPE_* (eq, ek) */
   float   sm_scale;
-  int32_t flags;          /* reserved, must be 0 */
+  int32_t flags;          /* FA_FLAG_* bits, 0 for the reference's launch sequence */
   /* Two more causal masks on the same machinery (no counterpart in the reference, whose README.md:17-18
      names such masks as the extension point); 0 = off; both need causal != 0 and exclude each other:
        window > 0 : sliding window -- row i sees only the last `window` keys up to its diagonal:
@@ -158,7 +164,7 @@ int fa_bwd_delta(const fa_params* p, void* stream);
 /* dk, dv summed over each group's query heads (needs lse, delta). */
 int fa_bwd_dkdv(const fa_params* p, void* stream);
 
-/* dq (needs lse, delta). */
+/* dq (needs lse, and delta unless FA_FLAG_DQ_DELTA is set). */
 int fa_bwd_dq(const fa_params* p, void* stream);
 
 /* Write keep(i,j) as one byte (0/1) per element into out[B,H,M,N] (contiguous),

@@ -70,7 +70,9 @@ def test_validate_codes():
     p = _good_params(buf); p.score_mode = 1; assert v(p) == -7     # doc mode without ids
     p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
-    p = _good_params(buf); p.flags = 1; assert v(p) == -7
+    p = _good_params(buf); p.flags = 2; assert v(p) == -7
+    p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; assert v(p) == 0 and v(p, 1) == 0
+    p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p, 1) == -10
     # sliding window / prefix: causal only, not both, not negative
     p = _good_params(buf); p.window = 64; assert v(p) == 0
     p = _good_params(buf); p.prefix = 64; assert v(p) == 0

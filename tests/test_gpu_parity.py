@@ -275,6 +275,51 @@ def test_graph_capture_and_replay():
             assert torch.equal(got, w_), (rep, name)
 
 
+@pytest.mark.parametrize("M,D,doc,dtype", [(2304, 64, True, torch.bfloat16), (450, 128, False, torch.float16),
+                                           (1000, 128, True, torch.bfloat16), (333, 16, True, torch.float16)])
+def test_dq_computes_delta(M, D, doc, dtype):
+    """FA_FLAG_DQ_DELTA: fa_bwd_dq forms delta itself and leaves it for fa_bwd_dkdv; delta, dq, dk, dv
+    must agree with the three-launch sequence (delta is a sum of the same products in another order:
+    1e-5 relative; the gradients then differ by a rounding of the 16-bit outputs at most)."""
+    import ctypes
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    L = _cabi.lib()
+    B, H = 2, 4
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(M + D)
+    rng = np.random.default_rng(M + D)
+    ids = torch.from_numpy(_ids(rng, B, H, M, "uniform")).to(dev)[:, None, :].expand(B, H, M) if doc else None
+    q, k, v, do = (torch.randn(B, H, M, D, generator=g).to(dtype).to(dev) for _ in range(4))
+    o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    lse = torch.empty(B, H, M, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    plan = _Plan(q, k, v, True, 1.0 / math.sqrt(D), ids, ids, 1 if doc else 0)
+    p = plan.p
+    p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+        _set4(getattr(p, f), t)
+    plan.ensure_workspace(dev)
+    ref, s = ctypes.byref(p), _stream_ptr(dev)
+    print("case dq computes delta", M, D, doc, dtype, flush=True)
+    for name in (["fa_mask_plan"] if doc else []) + ["fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"]:
+        _cabi.check(getattr(L, name)(ref, s), name)
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (delta, dq, dk, dv)]
+    for t in (delta, dq, dk, dv):
+        t.fill_(float("nan"))
+    p.flags = _cabi.FA_FLAG_DQ_DELTA
+    for name in ("fa_bwd_dq", "fa_bwd_dkdv"):
+        _cabi.check(getattr(L, name)(ref, s), name)
+    torch.cuda.synchronize()
+    assert torch.allclose(delta, want[0], rtol=1e-5, atol=1e-5 * float(want[0].abs().max())), (delta - want[0]).abs().max()
+    for name, got, w_ in zip(("dq", "dk", "dv"), (dq, dk, dv), want[1:]):
+        assert not torch.isnan(got).any(), name
+        err = (got.float() - w_.float()).abs().max().item()
+        assert err <= 2.0 ** -7 * max(1.0, w_.float().abs().max().item()), (name, err)
+
+
 def test_harness_cell_runs_and_agrees():
     from flash_mi355 import harness as Hn
     torch.manual_seed(5)

@@ -50,7 +50,8 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if (p->H % p->Hk != 0) return FA_ERR_SHAPE;
   if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
   if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC) return FA_ERR_MODE;
-  if (p->flags != 0) return FA_ERR_MODE;
+  if ((p->flags & ~FA_FLAG_DQ_DELTA) != 0) return FA_ERR_MODE;
+  if ((p->flags & FA_FLAG_DQ_DELTA) != 0 && p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
   if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
@@ -114,6 +115,7 @@ static KArgs make_args(const fa_params* p) {
   a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
   a.nQs = a.nKs = a.Pp = 0;
   a.qk_same = 0;
+  a.dq_delta = (p->flags & FA_FLAG_DQ_DELTA) != 0;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     const WsLayout w = ws_layout(p);
     char* ws = reinterpret_cast<char*>(p->workspace);

@@ -58,7 +58,9 @@ void bwd_dq_kernel(const KArgs a) {
   const T* dop = reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs;
   T* dqp = reinterpret_cast<T*>(a.dq) + b * a.dq_bs + h * a.dq_hs;
   const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
-  const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+  float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
+  const T* op = reinterpret_cast<const T*>(a.o) + b * a.o_bs + h * a.o_hs;
+  const bool own_delta = a.dq_delta != 0;   // delta = rowsum(O * dO) is computed here instead of being read
 
   vec8 qf[KS], dof[KS];
 #pragma unroll
@@ -66,9 +68,14 @@ void bwd_dq_kernel(const KArgs a) {
     qf[ks] = *reinterpret_cast<const vec8*>(qp + int64_t(rowc) * a.q_rs + ks * 16 + g * 8);
     dof[ks] = *reinterpret_cast<const vec8*>(dop + int64_t(rowc) * a.do_rs + ks * 16 + g * 8);
   }
+  vec8 of[KS] = {};
+  if (own_delta) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) of[ks] = *reinterpret_cast<const vec8*>(op + int64_t(rowc) * a.o_rs + ks * 16 + g * 8);
+  }
   const float c = a.scale_log2e;
   float L_i = lsep[rowc];
-  float delta_i = delp[rowc];
+  float delta_i = own_delta ? 0.f : delp[rowc];
 
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
   auto dec = [&](int t, const IdSummary& ks) { return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi), 0); };
@@ -80,6 +87,16 @@ void bwd_dq_kernel(const KArgs a) {
   for (int ks = 0; ks < KS; ++ks) { settle(qf[ks]); settle(dof[ks]); }
   settle(L_i);
   settle(delta_i);
+  if (own_delta) {
+    // the lane and its partner (lane ^ 32) hold the two halves of every 16 columns of the row
+    float part = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) part += float(of[ks][t]) * float(dof[ks][t]);
+    delta_i = xhalf_sum(part);
+    if (row >= 0 && g == 0 && wk.split == 0) delp[row] = delta_i;   // for the dk/dv kernel
+  }
   if (L_i == -INFINITY) L_i = INFINITY;  // row without any kept key: P = exp2(-inf) = 0
 
   TileLoader<DL, BN, D> ldK, ldV;

@@ -242,6 +242,7 @@ struct KArgs {
   int pfx_m1;   // prefix-LM: keys j <= pfx_m1 are seen by every row (-1: no prefix)
   int Pp;                 // entries of the permuted order per (b, h)
   int nQs, nKs;           // summary entries per (b, h)
+  int dq_delta;           // the dq kernel computes delta from O and dO itself and stores it
   int qk_same;            // eq and ek are one id vector (same pointer, strides and length): ksum also describes the rows
   float scale;            // sm_scale
   float scale_log2e;      // sm_scale * log2(e)

@@ -188,12 +188,19 @@ class _Impl:
             _set4(p.o_stride, o); _set4(p.do_stride, do)
             _set4(p.dq_stride, dq); _set4(p.dk_stride, dk); _set4(p.dv_stride, dv)
             stream = _stream_ptr(q.device)
-            _cabi.check(L.fa_bwd_delta(ctypes.byref(p), stream), "fa_bwd_delta")
-            if dlse is not None:
-                # dS = P * (dP - delta) + dLSE * P: a gradient arriving at LSE only shifts delta
-                delta.sub_(torch.where(torch.isinf(lse), torch.zeros_like(lse), dlse.to(torch.float32)))
-            _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
-            _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
+            if dlse is None and q.dtype != torch.float32:
+                # two launches instead of the reference's three (flash_triton.py:585-634): the dq kernel
+                # forms delta = rowsum(O * dO) from rows it holds anyway and leaves it for the dk/dv kernel
+                p.flags = _cabi.FA_FLAG_DQ_DELTA
+                _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
+                _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
+            else:
+                _cabi.check(L.fa_bwd_delta(ctypes.byref(p), stream), "fa_bwd_delta")
+                if dlse is not None:
+                    # dS = P * (dP - delta) + dLSE * P: a gradient arriving at LSE only shifts delta
+                    delta.sub_(torch.where(torch.isinf(lse), torch.zeros_like(lse), dlse.to(torch.float32)))
+                _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
+                _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
         return dq, dk, dv, None, None, None, None, None, None, None
 
 
