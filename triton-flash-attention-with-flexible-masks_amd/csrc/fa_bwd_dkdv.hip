@@ -27,9 +27,6 @@
 #ifndef FA_KV_PRE2
 #define FA_KV_PRE2 3
 #endif
-#ifndef FA_KV_FLAGSYNC
-#define FA_KV_FLAGSYNC 1
-#endif
 
 namespace fa {
 
@@ -223,112 +220,8 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
 
-  // One query tile.  BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute_split = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
-    const char* lqt = smem + BUF * TILE_BYTES;
-    const char* ldo = smem + (2 + BUF) * TILE_BYTES;
-    const char* aux = smem + AUX_OFF + BUF * AUX_BYTES;
-    const char* t1 = role == 0 ? lqt : ldo;   // rows operand of the first product
-    const char* t2 = role == 0 ? ldo : lqt;   // transposed operand of the second product
-    const int m0 = cur * BQ;  // natural order only
-
-    // wave-level decisions (identical for the two waves of a pair), taken by the tile iterator
-    const bool skip = (flags & TF_SKIP) != 0;
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      char* pbuf = smem + P_OFF + (qb * NKB + kb) * P_BYTES + lane * 16;
-      f32x16 x = zero;
-      vec8 yf[2] = {};   // P (score wave) or dS (gradient wave) of this block, rounded to the element type
-      if (!skip) {
-        // first product: S (score wave) or dP (gradient wave); operand rows a few LDS reads ahead
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 ra = lds_row8<E>(t1 + lo.row[ks] + qb * 32 * DL * 2);
-          x = E::mfma32(ra, frag[ks], x);
-        }
-        {
-          constexpr int PRE = KS < FA_KV_PRE ? KS : FA_KV_PRE;
-          __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
-#pragma unroll
-          for (int i = 0; i < KS - PRE; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          }
-          __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (role == 0) {
-          // S -> P for this lane's 16 query rows of the block
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            const int i0 = 32 * qb + 8 * q4 + 4 * g;  // row inside the tile
-            const f32x4 Lv = *reinterpret_cast<const f32x4*>(aux + i0 * 4);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) x[4 * q4 + t] = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
-          }
-          mask_p(x, qb, flags, tile_id, m0, aux);
-          // round P for the second product and hand the rounded values to the gradient wave of the
-          // pair (same lane, same register order)
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-#pragma unroll
-            for (int t = 0; t < 8; t += 2) {
-              const typename E::vec2 pr = E::cvt2(x[8 * half + t], x[8 * half + t + 1]);
-              yf[half][t] = pr[0]; yf[half][t + 1] = pr[1];
-            }
-            *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[half];
-          }
-        }
-      }
-      __syncthreads();
-      if (!skip) {
-        if (role == 1) {
-          // dS = P * (dP - delta), rounded for the second product
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const f32x8 pv = __builtin_convertvector(*reinterpret_cast<const vec8*>(pbuf + half * 1024), f32x8);
-#pragma unroll
-            for (int q2 = 0; q2 < 2; ++q2) {
-              const int i0 = 32 * qb + 8 * (2 * half + q2) + 4 * g;
-              const f32x4 dl = *reinterpret_cast<const f32x4*>(aux + 256 + i0 * 4);
-#pragma unroll
-              for (int t = 0; t < 4; t += 2) {
-                const int e = 4 * q2 + t;
-                const typename E::vec2 pr = E::cvt2(pv[e] * (x[8 * half + e] - dl[t]), pv[e + 1] * (x[8 * half + e + 1] - dl[t + 1]));
-                yf[half][e] = pr[0]; yf[half][e + 1] = pr[1];
-              }
-            }
-          }
-        }
-        // second product: dV^T += dO^T P (score wave) or dK^T += Q^T dS (gradient wave)
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int goff = (2 * qb + half) * 16 * DL * 2;
-#pragma unroll
-          for (int db = 0; db < DBN; ++db) {
-            const vec8 tf = lds_tr8<E>(t2 + lo.tr[db][0] + goff, t2 + lo.tr[db][1] + goff);
-            acc[db] = E::mfma32(tf, yf[half], acc[db]);
-          }
-        }
-        // transposed fragments (two reads each) a few MFMAs ahead, conversions just in time
-        {
-          constexpr int NM = 2 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
-          __builtin_amdgcn_sched_group_barrier(0x100, 2 * PRE, 0);
-#pragma unroll
-          for (int i = 0; i < NM; ++i) {
-            if (i % DBN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < NM - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  };
-
-  // The same tile with the two roles synchronised pairwise instead of by workgroup barriers: the
+  // One query tile, D > 64 (BUF is a compile-time constant so every LDS address is base + immediate).
+  // The two roles are synchronised pairwise, not by workgroup barriers: the
   // score wave publishes P of a 32-row block in LDS and then a sequence number; the gradient wave of
   // the pair polls that number.  LDS operations of one wave are executed in issue order, so the
   // number is never visible before P.  Waves of different key blocks drift apart inside a tile
@@ -539,8 +432,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     }
   };
   auto compute = [&](const int BUF, const int cur, const int flags, const int tile_id) __attribute__((always_inline)) {
-    if constexpr (SPLIT && FA_KV_FLAGSYNC) compute_flag(BUF, cur, flags, tile_id);
-    else if constexpr (SPLIT) compute_split(BUF, cur, flags, tile_id);
+    if constexpr (SPLIT) compute_flag(BUF, cur, flags, tile_id);
     else compute_both(BUF, cur, flags, tile_id);
   };
 
