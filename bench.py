@@ -48,8 +48,8 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {
     # bytes per launch: FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (factors from a 1 GiB copy in the same runs)
     ("cfg4_doc_causal_16k", "fa_bwd_dkdv"): 816_500_000,
-    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_562_000_000,
-    ("cfg4_doc_causal_16k", "fa_fwd"): 1_254_000_000,
+    ("cfg4_doc_causal_16k", "fa_bwd_dq"): 1_577_000_000,
+    ("cfg4_doc_causal_16k", "fa_fwd"): 1_264_000_000,
 }
 
 
@@ -82,8 +82,10 @@ def make_inputs(w, torch):
     return q, k, v, do, eq, ek
 
 
-def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
-    """Mean duration (ms) of every kernel of the step, each launched alone through the C ABI."""
+def time_kernels(w, q, k, v, do, eq, ek, torch, iters=20, warm=5):
+    """Duration (ms) of every kernel of the step, each launched alone through the C ABI, `iters` launches
+    back to back after `warm` untimed ones with a HIP event on the launch stream between any two
+    (the method of testing.py:140-152).  Returns the means and, under "_quantiles", (p20, median, p80)."""
     from flash_mi355 import _cabi
     from flash_mi355.api import _Plan, _set4, _stream_ptr
     L = _cabi.lib()
@@ -113,18 +115,21 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=10):
         names = [("fa_fwd", L.fa_fwd), ("fa_bwd_dq", L.fa_bwd_dq), ("fa_bwd_dkdv", L.fa_bwd_dkdv)]
     if w.doc:
         names.insert(0, ("fa_mask_plan", L.fa_mask_plan))
+    quant = {}
     for name, fn in names:
-        for _ in range(3):
+        for _ in range(warm):
             _cabi.check(fn(ref, stream), name)
         torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
+        ev[0].record()
+        for i in range(iters):
             fn(ref, stream)
-        e1.record()
-        e1.synchronize()
-        out[name] = e0.elapsed_time(e1) / iters
+            ev[i + 1].record()
+        ev[-1].synchronize()
+        ts = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(iters))
+        out[name] = ev[0].elapsed_time(ev[-1]) / iters
+        quant[name] = [round(ts[int(f * (iters - 1))], 4) for f in (0.2, 0.5, 0.8)]
+    out["_quantiles"] = quant
     return out
 
 
@@ -210,7 +215,8 @@ def main():
     def tf(flops, ms):
         return flops / ms * 1e-9
 
-    detail = {"ms": {n: round(t, 4) for n, t in kt.items()},
+    quantiles = kt.pop("_quantiles")
+    detail = {"ms": {n: round(t, 4) for n, t in kt.items()}, "ms_p20_p50_p80": quantiles,
               "tiles_nonempty": tiles, "tiles_total": total_tiles,
               "kept_fraction": round(kept / (w.B * w.Lq * w.Lk), 5)}
     for conv in ("tile", "dense", "elem"):
