@@ -458,9 +458,44 @@ def test_varlen_matches_per_sequence_oracle(causal):
             assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), f"sequence {s} {name} err {err}"
 
 
-def test_varlen_cross_attention_and_refusal():
+def test_varlen_causal_with_longer_key_sequences():
+    """Causal packed batch whose sequences have more keys than queries (chunked prefill / decoding):
+    every sequence bottom-right aligned on its own, against the oracle run on that sequence alone."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    lq, lk = [40, 3, 0, 100, 1], [40, 200, 5, 164, 77]
+    cuq = torch.tensor(np.concatenate([[0], np.cumsum(lq)]), dtype=torch.int32)
+    cuk = torch.tensor(np.concatenate([[0], np.cumsum(lk)]), dtype=torch.int32)
+    Tq, Tk, H, Hk, D = int(cuq[-1]), int(cuk[-1]), 4, 2, 64
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(Tq, H, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(Tk, Hk, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(Tk, Hk, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(Tq, H, D, generator=g).to(torch.bfloat16)
+    print("varlen causal, longer key sequences", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cuq.cuda(), cuk.cuda(), causal=True)
+    assert out.shape == (Tq, H, D)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for s in range(len(lq)):
+        a, b, c, d = int(cuq[s]), int(cuq[s + 1]), int(cuk[s]), int(cuk[s + 1])
+        if a == b:
+            assert kd.grad[c:d].abs().max().item() == 0 and vd.grad[c:d].abs().max().item() == 0   # keys nobody asked for
+            continue
+        sq = lambda t: t[a:b].transpose(0, 1)[None]
+        sk = lambda t: t[c:d].transpose(0, 1)[None]
+        ro, _, rdq, rdk, rdv = O.attention_autograd(sq(q), sk(k), sk(v), sq(do), True, None, None, None, 0)
+        for name, got, ref, sl in (("o", out.detach(), ro, sq), ("dq", qd.grad, rdq, sq), ("dk", kd.grad, rdk, sk), ("dv", vd.grad, rdv, sk)):
+            err = (sl(got.float().cpu()) - ref).abs().max().item()
+            assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), f"sequence {s} {name} err {err}"
+    with pytest.raises(AssertionError):   # fewer keys than queries in a sequence
+        attention_varlen(qd, kd, vd, cuq.cuda(), torch.tensor([0, 10, 240, 245, 409, 486], dtype=torch.int32).cuda(), causal=True)
+
+
+def test_varlen_cross_attention():
     """Different query and key boundaries (non-causal): each query sequence sees the keys of the
-    sequence with the same number; the causal form of that case is refused."""
+    sequence with the same number."""
     from flash_mi355 import attention_varlen
     from oracle import attention_oracle as O
     lq, lk = [40, 3, 100], [17, 200, 64]
@@ -481,8 +516,6 @@ def test_varlen_cross_attention_and_refusal():
         ro, _ = O.attention_closed_form(qs, ks, vs, False, None, None, None, 0)
         got = out[int(cuq[s]):int(cuq[s + 1])].transpose(0, 1)[None].float().cpu()
         assert (got - ro).abs().max().item() <= TOL_O
-    with pytest.raises(NotImplementedError):
-        attention_varlen(q.cuda(), k.cuda(), v.cuda(), cuq.cuda(), cuk.cuda(), causal=True)
 
 
 # fp32 tensors run on fp32 MFMAs: the oracle is fp32 too, so the bound is a few ulps of the

@@ -261,6 +261,25 @@ def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
     return (-(seq + 1)).to(torch.int32)
 
 
+def _varlen_causal_by_sequence(q, k, v, cu_seqlens_q, cu_seqlens_k, sm_scale, window):
+    """Causal packed batch whose query and key boundaries differ: one operator call per sequence on
+    [1, H, len, D] views of the packed tensors (bottom-right aligned, so a sequence needs at least
+    as many keys as queries, flash_triton.py:520)."""
+    assert cu_seqlens_q.shape == cu_seqlens_k.shape, "cu_seqlens_q and cu_seqlens_k must describe the same sequences"
+    cq, ck = cu_seqlens_q.tolist(), cu_seqlens_k.tolist()
+    assert cq[0] == 0 and ck[0] == 0 and cq[-1] == q.shape[0] and ck[-1] == k.shape[0], "cu_seqlens must span the packed tensors"
+    outs = []
+    for s in range(len(cq) - 1):
+        qs = q[cq[s]:cq[s + 1]]
+        if qs.shape[0] == 0:
+            continue
+        ks, vs = k[ck[s]:ck[s + 1]], v[ck[s]:ck[s + 1]]
+        assert ks.shape[0] >= qs.shape[0], f"sequence {s}: causal attention needs at least as many keys as queries"
+        q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (qs, ks, vs))
+        outs.append(attention(q4, k4, v4, True, sm_scale, window=window).squeeze(0).transpose(0, 1))
+    return torch.cat(outs, 0) if outs else torch.empty_like(q)
+
+
 def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_scale=None, *, window=0):
     """Packed variable-length batch (the calling convention of varlen flash-attention kernels):
     q [total_q, H, D], k and v [total_k, Hk, D], cu_seqlens_* int tensors [S+1] of cumulative
@@ -269,16 +288,19 @@ def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_
 
     The packed batch IS the document mask of the operator: one (batch) row of total_* tokens whose
     ids are the negated sequence numbers, so no padding and no copy -- q, k, v are passed as
-    [1, H, total, D] views.  causal=True needs cu_seqlens_k to be cu_seqlens_q (self-attention,
-    where the causal bound of the packed row and of every sequence coincide); with different
-    boundaries the per-sequence bottom-right alignment is not a single offset and is refused.
+    [1, H, total, D] views.  That holds for every non-causal case and for causal self-attention
+    (cu_seqlens_k equal to cu_seqlens_q: the causal bound of the packed row and of every sequence
+    coincide).  Causal with different boundaries (queries that are the tail of a longer key
+    sequence: chunked prefill, decoding) aligns every sequence bottom-right on its own, which is
+    not one offset of the packed row: those sequences are launched one by one, each as the
+    rectangular causal case of the operator (flash_triton.py:520-521), still without a copy.
     (No counterpart in the reference, which takes eq/ek directly, flash_triton.py:506.)"""
     assert q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be [total, heads, D]"
     same = cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q
     if not same and causal:
         same = cu_seqlens_k.shape == cu_seqlens_q.shape and bool(torch.equal(cu_seqlens_k, cu_seqlens_q))
         if not same:
-            raise NotImplementedError("causal attention over packed sequences needs cu_seqlens_k == cu_seqlens_q")
+            return _varlen_causal_by_sequence(q, k, v, cu_seqlens_q, cu_seqlens_k, sm_scale, window)
     Tq, H, _ = q.shape
     Tk = k.shape[0]
     eq = varlen_ids(cu_seqlens_q, Tq)
