@@ -57,7 +57,7 @@ extern "C" {
 #define FA_DTYPE_FP16 1
 #define FA_DTYPE_FP32 2   /* fp32 tensors: fp32 MFMA throughout (the reference takes fp32 like any float type) */
 #define FA_IDTYPE_I32 0
-#define FA_IDTYPE_I64 1
+#define FA_IDTYPE_I64 1   /* values must fit in int32: fa_mask_plan narrows them with saturation */
 
 /* return codes */
 #define FA_OK                    0
