@@ -84,11 +84,17 @@ void bwd_dkdv_kernel(const KArgs a) {
     const T* vsrc = reinterpret_cast<const T*>(a.v) + b * a.v_bs + hk * a.v_hs + int64_t(keyc) * a.v_rs;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) frag2[ks] = *reinterpret_cast<const vec8*>(vsrc + ks * 16 + g * 8);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) settle(frag2[ks]);
   }
+  // Where to wait for these fragments.  The 64-key role-split form serves short tile streams: only
+  // right before the tile loop, so that the set-up below overlaps their flight (3 % of the kernel at
+  // 16 query tiles per workgroup, under 1 % at a dozen).  The other forms wait here: for the
+  // 128-key form, which serves long streams, that gave the faster loop (4.24 against 4.39 ms, plain
+  // causal 16K); at D <= 64 the difference stayed inside the run-to-run spread.
+  constexpr bool LATE_SETTLE = SPLIT && NKB == 2;
+  if (!LATE_SETTLE) {
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) settle(frag[ks]);
+    for (int ks = 0; ks < KS; ++ks) { settle(frag[ks]); if (!SPLIT) settle(frag2[ks]); }
+  }
   const float c = a.scale_log2e;
   // rows that may see this lane's key: [row_lo, row_lo + row_span)
   // (causal: from the diagonal on, or from row 0 for a key of the prefix; sliding window: `win` rows)
@@ -508,6 +514,12 @@ void bwd_dkdv_kernel(const KArgs a) {
       if (DOC) fetch_idx(cur);
       load_tile(cur, 0);
       if (DOC && nxt >= 0) fetch_idx(nxt);
+    }
+    if (LATE_SETTLE && gi == 0) {
+      // the K / V fragments are complete before the tile loop (their wait would otherwise sit at the
+      // first use inside it)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) settle(frag[ks]);
     }
     while (cur >= 0) {
       int nxt2 = -1, nxt2_fl = 0, nxt2_id = 0;
