@@ -188,6 +188,29 @@ def test_lse_output_is_differentiable():
         assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
 
 
+@pytest.mark.parametrize("use", ["out", "lse"])
+def test_lse_entry_point_with_one_result_used(use):
+    """Only one of (O, LSE) enters the loss: the other one's gradient arrives as None."""
+    from flash_mi355 import attention_with_lse
+    from oracle import attention_oracle as O
+    B, H, L, D = 1, 2, 200, 64
+    g = torch.Generator().manual_seed(37)
+    q, k, v, do = (torch.randn(B, H, L, D, generator=g).to(torch.float16) for _ in range(4))
+    w = torch.randn(B, H, L, generator=g)
+    print("case lse entry point, used:", use, flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out, lse = attention_with_lse(qd, kd, vd, True)
+    loss = (out.float() * do.cuda().float()).sum() if use == "out" else (lse * w.cuda()).sum()
+    loss.backward()
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    ro, rl = O.attention_closed_form(qr, kr, vr, True, None, None, None, 0)
+    ((ro * do.float()).sum() if use == "out" else (rl * w).sum()).backward()
+    for name, got, want in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        want = torch.zeros_like(got, dtype=torch.float32, device="cpu") if want is None else want   # LSE does not depend on v
+        err = (got.float().cpu() - want).abs().max().item()
+        assert err <= TOL_O * max(1.0, want.abs().max().item() / 4), (name, err)
+
+
 @pytest.mark.parametrize("seed", list(range(100, 124)))
 def test_random_shapes(seed):
     """Seeded draws over the whole argument space of the operator: head size, head counts and groups,

@@ -171,6 +171,8 @@ class _Impl:
         B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
         score_func_mode, window, prefix = ctx.score_func_info
         L = _cabi.lib()
+        if do is None:   # only LSE was used
+            do = torch.zeros_like(o)
         do = _aligned(maybe_contiguous(do))
         with torch.cuda.device(q.device):
             plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix)
@@ -227,6 +229,7 @@ class FlashAttentionWithLse(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
         out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
+        ctx.set_materialize_grads(False)   # a result that is not used arrives as None, not as zeros
         return out, lse * math.log(2.0)
 
     @staticmethod
