@@ -79,6 +79,8 @@ def make_inputs(w, torch):
     if w.doc:  # ids shared by the heads, passed head-expanded as the reference harness does (testing.py:118)
         eq = torch.from_numpy(w.eq).to(dev)[:, None, :].expand(w.B, w.H, w.Lq)
         ek = torch.from_numpy(w.ek).to(dev)[:, None, :].expand(w.B, w.H, w.Lk)
+    if w.block is not None:   # block mask: the byte map travels in the place of eq (score mode 2)
+        eq = ek = torch.from_numpy(w.block).to(dev)[:, None].expand(w.B, w.H, *w.block.shape[1:]).to(torch.uint8)
     return q, k, v, do, eq, ek
 
 
@@ -90,7 +92,7 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=20, warm=5):
     from flash_mi355.api import _Plan, _set4, _stream_ptr
     L = _cabi.lib()
     dev = q.device
-    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else 0, w.window, w.prefix)
+    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else (2 if w.block is not None else 0), w.window, w.prefix)
     p = plan.p
     o = torch.empty_like(q)
     lse = torch.empty(w.B, w.H, w.Lq, device=dev, dtype=torch.float32)
@@ -180,7 +182,7 @@ def main():
 
     w = W.make_workload(args.workload)
     q, k, v, do, eq, ek = make_inputs(w, torch)
-    mode = 1 if w.doc else 0
+    mode = 1 if w.doc else (2 if w.block is not None else 0)
     scale = 1.0 / math.sqrt(w.D)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
 
@@ -245,12 +247,12 @@ def main():
 
     value = tf(3.5 * f_fwd["tile"], ms_per_step)
     line = {
-        "metric": f"attention fwd+bwd TFLOP/s ({w.dtype}, {'doc+' if w.doc else ''}{'causal' if w.causal else 'no'} mask, tile-effective FLOPs)",
+        "metric": f"attention fwd+bwd TFLOP/s ({w.dtype}, {'doc+' if w.doc else ''}{'block+' if w.block is not None else ''}{'causal' if w.causal else 'no'} mask, tile-effective FLOPs)",
         "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": w.name, "B": w.B, "H": w.H, "Hk": w.Hk, "Lq": w.Lq, "Lk": w.Lk, "D": w.D,
-                   "causal": w.causal, "doc_mask": w.doc},
+                   "causal": w.causal, "doc_mask": w.doc, "block_mask": w.block is not None},
         "pct_of_mfma_peak": round(100 * value / peak, 2),
         "detail": detail, "roofline": roofline,
     }

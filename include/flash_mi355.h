@@ -46,11 +46,18 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 3
+#define FA_ABI_VERSION 4
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
 #define FA_SCORE_MODE1_DOC  1
+/* Block mask (no counterpart in the reference, whose README.md:17-18 names block-sparse patterns as the
+   extension point): `eq` points to bytes [B, H, ceil(M/64), ceil(N/64)], eq_stride = its batch, head
+   and row strides in bytes (0 allowed for batch and head), the column stride is 1; `ek`, `id_dtype`
+   and the workspace are not used and fa_mask_plan is not needed.  A pair (i, j) is kept iff the byte of
+   block (i / 64, j / 64) is non-zero and the causal / window / prefix terms hold.  bf16 / fp16 only. */
+#define FA_SCORE_MODE2_BLOCK 2
+#define FA_MASK_BLOCK 64
 
 /* element types */
 #define FA_DTYPE_BF16 0

@@ -49,6 +49,8 @@ import torch
 
 SCORE_FUNC_MODE0_NOPE = 0  # flash_triton.py:20
 SCORE_FUNC_MODE1_DOC = 1   # flash_triton.py:22
+SCORE_FUNC_MODE2_BLOCK = 2  # the library's block mask (no counterpart in the reference): eq = [B|1, H|1, ceil(Lq/64), ceil(Lk/64)]
+MASK_BLOCK = 64
 LOG2E = 1.4426950408889634
 
 
@@ -82,6 +84,13 @@ def keep_mask(Lq: int, Lk: int, causal: bool, eq=None, ek=None,
         assert eq.ndim == 3 and ek.ndim == 3
         doc = (eq[..., :, None] >= 0) | (eq[..., :, None] == ek[..., None, :])
         keep = keep & doc
+    elif score_func_mode == SCORE_FUNC_MODE2_BLOCK:
+        # keep iff the block (i // 64, j // 64) is switched on; eq carries the block map, ek is not used
+        bm = np.asarray(eq) != 0
+        assert bm.ndim == 4 and bm.shape[2] == -(-Lq // MASK_BLOCK) and bm.shape[3] == -(-Lk // MASK_BLOCK)
+        i = np.arange(Lq) // MASK_BLOCK
+        j = np.arange(Lk) // MASK_BLOCK
+        keep = keep & bm[:, :, i[:, None], j[None, :]]
     elif score_func_mode != SCORE_FUNC_MODE0_NOPE:
         raise ValueError(f"unknown score_func_mode {score_func_mode}")
     return keep

@@ -128,6 +128,63 @@ def test_mask_bit_exact():
         assert np.array_equal(got, ref)
 
 
+BLOCK_CASES = [
+    # B, H, Hk, M, N, D, dtype, causal, window, density, broadcast (block map shared by batch and heads)
+    (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 0, 0.5, False),
+    (2, 2, 2, 512, 512, 128, torch.bfloat16, True, 0, 0.5, False),
+    (1, 4, 2, 450, 700, 128, torch.float16, True, 0, 0.6, True),      # grouped, ragged, rectangular
+    (1, 2, 2, 300, 300, 64, torch.bfloat16, True, 0, 0.4, False),
+    (1, 2, 1, 333, 520, 64, torch.float16, False, 0, 0.3, True),
+    (1, 2, 2, 200, 200, 16, torch.bfloat16, True, 0, 0.5, False),
+    (1, 2, 2, 640, 640, 32, torch.bfloat16, False, 0, 0.2, False),
+    (1, 1, 1, 2304, 2304, 128, torch.bfloat16, True, 0, 0.3, False),   # long stream: the 128-key dk/dv form
+    (1, 2, 2, 1024, 1024, 128, torch.bfloat16, True, 300, 0.7, False),  # with a sliding window
+    (1, 2, 2, 192, 192, 128, torch.bfloat16, False, 0, 0.0, False),    # nothing kept at all
+]
+
+
+@pytest.mark.parametrize("case", BLOCK_CASES, ids=lambda c: "blk-B%d-H%d_%d-M%d-N%d-D%d-c%d-w%d" % (
+    c[0], c[1], c[2], c[3], c[4], c[5], c[7], c[8]))
+def test_block_mask_parity(case):
+    """Block-sparse attention (64 x 64 blocks switched on and off by a byte map): mask bit-exact, O, LSE
+    and the gradients against the oracle; rows whose blocks are all off give O = 0, LSE = -inf, no gradient."""
+    from flash_mi355 import attention_with_lse, attention, mask_dump, SCORE_FUNC_MODE2_BLOCK
+    from oracle import attention_oracle as O
+    B, H, Hk, M, N, D, dtype, causal, window, density, shared = case
+    rng = np.random.default_rng(M * 7 + N + D)
+    g = torch.Generator().manual_seed(M + N + D)
+    nbr, nbc = -(-M // 64), -(-N // 64)
+    bm = torch.from_numpy((rng.random((1 if shared else B, 1 if shared else H, nbr, nbc)) < density))
+    if density > 0:
+        bm[..., 0, :] = False          # a row of blocks with nothing kept
+    q = torch.randn(B, H, M, D, generator=g).to(dtype)
+    k = torch.randn(B, Hk, N, D, generator=g).to(dtype)
+    v = torch.randn(B, Hk, N, D, generator=g).to(dtype)
+    do = torch.randn(B, H, M, D, generator=g).to(dtype)
+    print(f"case block mask {case}", flush=True)
+    keep = mask_dump(B, H, M, N, causal, bm.cuda(), None, SCORE_FUNC_MODE2_BLOCK, window=window).cpu().numpy()
+    ref_keep = np.broadcast_to(O.keep_mask(M, N, causal, bm.numpy(), None, 2, window=window), (B, H, M, N))
+    assert np.array_equal(keep, ref_keep)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    with torch.no_grad():
+        out, lse = attention_with_lse(qd, kd, vd, causal, None, window=window, block_mask=bm.cuda())
+    ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, None, bm, None, 2, window=window)
+    dead = torch.isinf(ref_lse)
+    assert torch.equal(torch.isinf(lse.cpu()), dead)
+    if (~dead).any():
+        assert (lse.cpu()[~dead] - ref_lse[~dead]).abs().max().item() <= TOL_LSE
+    assert not torch.isnan(out).any()
+    assert (out.float().cpu() - ref_o).abs().max().item() <= TOL_O
+    out2 = attention(qd, kd, vd, causal, None, window=window, block_mask=bm.cuda())
+    out2.backward(do.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(out2.detach(), out)
+    for name, got, ref in (("dq", qd.grad, ref_dq), ("dk", kd.grad, ref_dk), ("dv", vd.grad, ref_dv)):
+        assert not torch.isnan(got).any(), name
+        err = (got.float().cpu() - ref).abs().max().item()
+        assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), f"{name} err {err}"
+
+
 def test_all_global_and_all_local_ids():
     _run_case(1, 2, 2, 256, 256, 128, torch.bfloat16, True, True, seed=5, ids_kind="allglobal")
     _run_case(1, 2, 2, 256, 256, 128, torch.bfloat16, True, True, seed=6, ids_kind="alllocal")

@@ -235,6 +235,44 @@ def test_eager_cpu_path_matches_closed_form():
     assert torch.allclose(got, ref, atol=1e-5)
 
 
+# ------------------------------------------------------------------ block mask
+def test_block_mask_brute_force_and_special_cases():
+    """keep(i, j) of the block mode against a double loop; an all-ones map changes nothing; a block-diagonal
+    map makes every 64-row block an attention problem of its own; the library routine with the same
+    boolean mask written out."""
+    rng = np.random.default_rng(3)
+    for (M, N, causal, window) in [(130, 200, True, 0), (64, 64, False, 0), (200, 130, False, 0), (190, 190, True, 70)]:
+        nbr, nbc = -(-M // 64), -(-N // 64)
+        bm = rng.integers(0, 2, (2, 3, nbr, nbc))
+        keep = np.broadcast_to(O.keep_mask(M, N, causal, bm, None, O.SCORE_FUNC_MODE2_BLOCK, window=window), (2, 3, M, N))
+        gap = max(0, N - M)
+        for b in range(2):
+            for h in range(3):
+                for i in range(0, M, 7):
+                    for j in range(N):
+                        want = bm[b, h, i // 64, j // 64] != 0
+                        if causal:
+                            want = want and gap + i >= j and (window == 0 or j > gap + i - window)
+                        assert keep[b, h, i, j] == want
+        ones = np.ones((1, 1, nbr, nbc), dtype=np.uint8)
+        assert np.array_equal(O.keep_mask(M, N, causal, ones, None, 2, window=window), O.keep_mask(M, N, causal, window=window))
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 2, 192, 32, generator=g) for _ in range(3))
+    eye = torch.eye(3, dtype=torch.bool)[None, None]
+    o, lse = O.attention_closed_form(q, k, v, False, None, eye, None, O.SCORE_FUNC_MODE2_BLOCK)
+    for blk in range(3):
+        sl = slice(64 * blk, 64 * blk + 64)
+        o1, l1 = O.attention_closed_form(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        assert torch.allclose(o[:, :, sl], o1, atol=1e-6) and torch.allclose(lse[:, :, sl], l1, atol=1e-6)
+    bm2 = torch.from_numpy(np.tril(np.ones((3, 3), bool))[None, None])
+    keep = torch.from_numpy(O.keep_mask(192, 192, True, bm2.numpy(), None, 2))
+    o2, _ = O.attention_closed_form(q, k, v, True, None, bm2, None, 2)
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=keep.expand(1, 2, 192, 192))
+    assert torch.allclose(o2, ref, atol=1e-5)
+    ref_causal = F.scaled_dot_product_attention(q, k, v, is_causal=True)   # lower-triangular blocks + causal = causal
+    assert torch.allclose(o2, ref_causal, atol=1e-5)
+
+
 # ------------------------------------------------------------------ sliding window / prefix-LM
 @pytest.mark.parametrize("M,N", [(9, 9), (5, 12), (1, 6)])
 def test_window_and_prefix_masks_brute_force(M, N):

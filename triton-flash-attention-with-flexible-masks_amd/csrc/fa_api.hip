@@ -49,7 +49,13 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if (p->B <= 0 || p->H <= 0 || p->Hk <= 0 || p->M <= 0 || p->N <= 0) return FA_ERR_SHAPE;
   if (p->H % p->Hk != 0) return FA_ERR_SHAPE;
   if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
-  if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC) return FA_ERR_MODE;
+  if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC && p->score_mode != FA_SCORE_MODE2_BLOCK)
+    return FA_ERR_MODE;
+  if (p->score_mode == FA_SCORE_MODE2_BLOCK) {
+    if (p->eq == nullptr) return FA_ERR_MODE;
+    if (p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
+    if (p->eq_stride[0] < 0 || p->eq_stride[1] < 0 || p->eq_stride[2] < (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK) return FA_ERR_STRIDE;
+  }
   if ((p->flags & ~FA_FLAG_DQ_DELTA) != 0) return FA_ERR_MODE;
   if ((p->flags & FA_FLAG_DQ_DELTA) != 0 && p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
@@ -79,13 +85,13 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
 }
 
 extern "C" uint64_t fa_workspace_bytes(const fa_params* p) {
-  if (p == nullptr || p->score_mode == FA_SCORE_MODE0_NOPE) return 0;
+  if (p == nullptr || p->score_mode != FA_SCORE_MODE1_DOC) return 0;
   if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
   return ws_layout(p).total;
 }
 
 extern "C" uint64_t fa_workspace_plan_bytes(const fa_params* p) {
-  if (p == nullptr || p->score_mode == FA_SCORE_MODE0_NOPE) return 0;
+  if (p == nullptr || p->score_mode != FA_SCORE_MODE1_DOC) return 0;
   if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
   return ws_layout(p).plan_bytes;
 }
@@ -116,6 +122,12 @@ static KArgs make_args(const fa_params* p) {
   a.nQs = a.nKs = a.Pp = 0;
   a.qk_same = 0;
   a.dq_delta = (p->flags & FA_FLAG_DQ_DELTA) != 0;
+  a.bmask = nullptr; a.bm_bs = a.bm_hs = a.bm_rs = 0;
+  a.nBr = (p->M + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK; a.nBc = (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK;
+  if (p->score_mode == FA_SCORE_MODE2_BLOCK) {
+    a.bmask = reinterpret_cast<const unsigned char*>(p->eq);
+    a.bm_bs = p->eq_stride[0]; a.bm_hs = p->eq_stride[1]; a.bm_rs = p->eq_stride[2];
+  }
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     const WsLayout w = ws_layout(p);
     char* ws = reinterpret_cast<char*>(p->workspace);
@@ -154,7 +166,7 @@ static int finish(int hip_rc) {
 extern "C" int fa_mask_plan(const fa_params* p, void* stream) {
   int rc = fa_validate(p, 2);
   if (rc != FA_OK) return rc;
-  if (p->score_mode == FA_SCORE_MODE0_NOPE) return FA_OK;
+  if (p->score_mode != FA_SCORE_MODE1_DOC) return FA_OK;
   return finish(launch_mask_plan(p, ws_layout(p), reinterpret_cast<hipStream_t>(stream)));
 }
 

@@ -245,7 +245,10 @@ __global__ __launch_bounds__(256) void mask_dump_kernel(const KArgs a, uint8_t* 
     eq_i = a.eq32[b * a.eq_bs + h * a.eq_hs + i];
     ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + j];
   }
-  out[(int64_t(bh) * a.M + i) * a.N + j] = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1) ? 1 : 0;
+  bool keep = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1);
+  if (!DOC && a.bmask != nullptr)
+    keep = keep && a.bmask[b * a.bm_bs + h * a.bm_hs + int64_t(i / FA_MASK_BLOCK) * a.bm_rs + j / FA_MASK_BLOCK] != 0;
+  out[(int64_t(bh) * a.M + i) * a.N + j] = keep ? 1 : 0;
 }
 
 int launch_mask_dump(const KArgs& a, bool causal, bool doc, uint8_t* out, hipStream_t s) {

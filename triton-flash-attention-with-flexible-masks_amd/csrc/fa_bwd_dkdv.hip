@@ -478,14 +478,26 @@ void bwd_dkdv_kernel(const KArgs a) {
       first = 0;
     }
     // decisions of this wave pair (keys nw .. nw+31) for query tile t, evaluated by the lane that tests the tile
+    // block mask: the byte column(s) of the workgroup's one or two 64-key blocks; a query tile is one
+    // row of blocks, a wave's 32 keys lie inside one block (no element mask needed)
+    const unsigned char* bmk = (!DOC && a.bmask != nullptr) ? a.bmask + b * a.bm_bs + h * a.bm_hs + n0 / 64 : nullptr;
     auto dec = [&](int t, const IdSummary& qs) {
-      bool skip, lim, doc = false, glob = false, col = false;
+      bool skip, lim, doc = false, glob = false, col = false, none = false;
       if (!DOC) {
         const int m0 = t * BQ;
         const int rmin = m0, rmax = min(m0 + BQ - 1, a.M - 1);
         skip = (nw >= a.N) || (CAUSAL && ((a.gap + rmax < nw && nw > a.pfx_m1) || a.gap + rmin - a.win + 1 > nw + 31));
         lim = (m0 + BQ > a.M) || (nw + 32 > a.N) ||
               (CAUSAL && ((a.gap + rmin < nw + 31 && nw + 31 > a.pfx_m1) || a.gap + rmax - a.win + 1 > nw));
+        if (bmk != nullptr) {
+          const bool in = t < a.nBr;
+          const unsigned char* r = bmk + int64_t(t) * a.bm_rs;
+          const unsigned b0 = in ? r[0] : 0u;
+          const unsigned b1 = (in && BK > 64 && n0 / 64 + 1 < a.nBc) ? r[1] : 0u;
+          const unsigned mine = (BK > 64 && kb >= 2) ? b1 : b0;
+          skip = skip || mine == 0;
+          none = (b0 | b1) == 0;
+        }
       } else {
         skip = (nw >= a.N) || (CAUSAL && ((a.gap + qs.rmax < nw && nw > a.pfx_m1) || a.gap + qs.rmin - a.win + 1 > nw + 31)) ||
                !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
@@ -498,7 +510,8 @@ void bwd_dkdv_kernel(const KArgs a) {
         col = doc && !glob && qs.lo == qs.hi;
         if (col) doc = false;
       }
-      return tile_value((skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0) | (col ? TF_COL : 0), qs.lo);
+      return tile_value((skip ? TF_SKIP : 0) | (lim ? TF_LIM : 0) | (doc ? TF_DOC : 0) | (glob ? TF_GLOB : 0) | (col ? TF_COL : 0) |
+                        (none ? TF_NONE : 0), qs.lo);
     };
     TileIter it;
     it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL && n0 > a.pfx_m1 ? n0 - a.gap : (int)0x80000000,

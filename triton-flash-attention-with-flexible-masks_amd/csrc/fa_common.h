@@ -243,6 +243,10 @@ struct KArgs {
   int Pp;                 // entries of the permuted order per (b, h)
   int nQs, nKs;           // summary entries per (b, h)
   int dq_delta;           // the dq kernel computes delta from O and dO itself and stores it
+  // block mask (FA_SCORE_MODE2_BLOCK): bytes [B, H, nBr, nBc] per 64 x 64 block of (row, key) pairs, or null
+  const unsigned char* bmask;
+  int64_t bm_bs, bm_hs, bm_rs;
+  int nBr, nBc;
   int qk_same;            // eq and ek are one id vector (same pointer, strides and length): ksum also describes the rows
   float scale;            // sm_scale
   float scale_log2e;      // sm_scale * log2(e)

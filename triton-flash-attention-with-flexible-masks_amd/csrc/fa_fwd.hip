@@ -79,7 +79,11 @@ void fwd_kernel(const KArgs a) {
     qf[ks] = *reinterpret_cast<const vec8*>(qp + int64_t(rowc) * a.q_rs + ks * 16 + g * 8);
 
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
-  auto dec = [&](int t, const IdSummary& ks) { return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi), 0); };
+  QBlockMask bmq;
+  bmq.init(a, b, h, wk.tile);
+  auto dec = [&](int t, const IdSummary& ks) {
+    return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi) | (DOC ? 0 : bmq.flags(t)), 0);
+  };
   TileIter it;
   it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);   // its summaries travel together with Q
 

@@ -180,6 +180,9 @@ FA_DEV typename E::vec8 lds_tr8(const char* p0, const char* p1) {
 // dec() returns the TF_ bits in its low word and, optionally, one value in its high word
 // (tile_value(): handed out as `value`, e.g. the single id of a tile).
 enum { TF_SKIP = 1, TF_LIM = 2, TF_DOC = 4, TF_GLOB = 8, TF_COL = 16, TF_NBITS = 5 };
+// Returned by dec() next to those, not handed out: no wave of the workgroup needs this candidate
+// (block mask), so it is not visited at all.
+enum { TF_NONE = 32 };
 FA_DEV long long tile_value(int flags, int value) { return (long long)(unsigned)flags | ((long long)value << 32); }
 
 struct TileIter {
@@ -224,6 +227,7 @@ struct TileIter {
     }
     const long long fv = dec(t, s);
     const int f = (int)fv;
+    v = v && (f & TF_NONE) == 0;
     c_val = (int)(fv >> 32);
 #pragma unroll
     for (int i = 0; i < TF_NBITS; ++i) fm[i] = __builtin_amdgcn_ballot_w64(((f >> i) & 1) != 0);
@@ -375,6 +379,30 @@ FA_DEV void mask_doc(f32x16& s, const char* ids, int eq_i, bool glob_i, float fi
     for (int t = 0; t < 4; ++t) s[4 * q4 + t] = (glob_i || ekv[q4][t] == eq_i) ? s[4 * q4 + t] : fill;
   }
 }
+
+// Block mask seen from a 128-row query tile of the forward / dq kernels (natural row order): the two
+// rows of 64 x 64 blocks the tile covers.  flags(t) are the TF_ bits the mask adds for key tile t
+// (64 keys = one block column): TF_SKIP when the block of this wave's rows is off, TF_NONE when
+// both are.  A wave's 32 rows and a tile's 64 keys lie inside one block, so no element mask is needed.
+struct QBlockMask {
+  const unsigned char* r0;   // null: no block mask
+  const unsigned char* r1;   // null: the tile's second half lies past the last row
+  int ncol;
+  FA_DEV void init(const KArgs& a, int b, int h, int tile) {
+    r0 = r1 = nullptr; ncol = a.nBc;
+    if (a.bmask == nullptr) return;
+    const unsigned char* base = a.bmask + b * a.bm_bs + h * a.bm_hs;
+    r0 = base + int64_t(2 * tile) * a.bm_rs;
+    if (2 * tile + 1 < a.nBr) r1 = base + int64_t(2 * tile + 1) * a.bm_rs;
+  }
+  FA_DEV int flags(int t) const {
+    if (r0 == nullptr) return 0;
+    const bool in = t < ncol;
+    const unsigned b0 = in ? r0[t] : 0u, b1 = (in && r1 != nullptr) ? r1[t] : 0u;
+    const unsigned mine = (threadIdx.x >> 7) ? b1 : b0;   // waves 0, 1: first half; waves 2, 3: second half
+    return (mine == 0 ? TF_SKIP : 0) | ((b0 | b1) == 0 ? TF_NONE : 0);
+  }
+};
 
 // ---------------------------------------------------------------------------
 // Work assignment of one workgroup of the forward / dq kernels, including the split of the

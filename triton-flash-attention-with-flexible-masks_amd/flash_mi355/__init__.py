@@ -5,7 +5,7 @@
 
 The four public names match the reference module ``flash_triton``.
 """
-from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, FlashAttention, FlashAttentionWithLse, attention,
+from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, SCORE_FUNC_MODE2_BLOCK, FlashAttention, FlashAttentionWithLse, attention,
                   attention_varlen, attention_with_lse, mask_dump, maybe_contiguous, varlen_ids)
 
 __all__ = ["attention", "FlashAttention", "FlashAttentionWithLse", "SCORE_FUNC_MODE0_NOPE", "SCORE_FUNC_MODE1_DOC",

@@ -11,9 +11,11 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libflash_mi355.so"
 
-FA_ABI_VERSION = 3
+FA_ABI_VERSION = 4
 FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
+FA_SCORE_MODE2_BLOCK = 2
+FA_MASK_BLOCK = 64
 FA_DTYPE_BF16 = 0
 FA_DTYPE_FP16 = 1
 FA_DTYPE_FP32 = 2

@@ -16,6 +16,7 @@ from . import _cabi
 
 SCORE_FUNC_MODE0_NOPE = 0  # flash_triton.py:20
 SCORE_FUNC_MODE1_DOC = 1   # flash_triton.py:22
+SCORE_FUNC_MODE2_BLOCK = 2  # block mask: set by the block_mask argument of attention(), no counterpart in the reference
 
 _DTYPES = {torch.bfloat16: _cabi.FA_DTYPE_BF16, torch.float16: _cabi.FA_DTYPE_FP16, torch.float32: _cabi.FA_DTYPE_FP32}
 _ID_DTYPES = {torch.int32: _cabi.FA_IDTYPE_I32, torch.int64: _cabi.FA_IDTYPE_I64}
@@ -64,7 +65,11 @@ class _Plan:
         p.flags = 0
         p.window, p.prefix = int(window), int(prefix)
         self.keep = [q, k, v]
-        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+        if score_func_mode == SCORE_FUNC_MODE2_BLOCK:   # eq is the block map [B, H, rows of blocks, columns of blocks], bytes
+            p.eq = eq.data_ptr()
+            _set3(p.eq_stride, eq)
+            self.keep += [eq]
+        elif score_func_mode != SCORE_FUNC_MODE0_NOPE:
             p.eq, p.ek = eq.data_ptr(), ek.data_ptr()
             _set3(p.eq_stride, eq); _set3(p.ek_stride, ek)
             p.id_dtype = _ID_DTYPES[eq.dtype]
@@ -130,7 +135,7 @@ class _Impl:
         if eq is None:
             assert score_func_mode == SCORE_FUNC_MODE0_NOPE
         # -- checks the reference leaves to the Triton launcher --
-        assert score_func_mode in (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC), "unknown score_func_mode"
+        assert score_func_mode in (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, SCORE_FUNC_MODE2_BLOCK), "unknown score_func_mode"
         window, prefix = int(window or 0), int(prefix or 0)
         assert window >= 0 and prefix >= 0 and not (window and prefix), "window and prefix exclude each other"
         assert causal or not (window or prefix), "window / prefix are causal masks"
@@ -138,7 +143,14 @@ class _Impl:
         assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, \
             "q, k, v must share one of torch.bfloat16 / torch.float16 / torch.float32"
         assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
-        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+        if score_func_mode == SCORE_FUNC_MODE2_BLOCK:
+            assert q.dtype != torch.float32, "block masks are implemented for bfloat16 / float16"
+            nbr, nbc = -(-M // _cabi.FA_MASK_BLOCK), -(-N // _cabi.FA_MASK_BLOCK)
+            assert eq.dim() == 4 and eq.shape[0] in (1, B) and eq.shape[1] in (1, H) and tuple(eq.shape[2:]) == (nbr, nbc), \
+                f"block_mask must be [bs|1, H|1, {nbr}, {nbc}] (blocks of 64 x 64)"
+            eq = maybe_contiguous((eq != 0).to(torch.uint8).to(q.device)).expand(B, H, nbr, nbc)
+            ek = eq
+        elif score_func_mode != SCORE_FUNC_MODE0_NOPE:
             eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
             if eq.dtype != ek.dtype:   # one id width per call
                 eq, ek = eq.to(torch.int64), ek.to(torch.int64)
@@ -237,11 +249,22 @@ class FlashAttentionWithLse(torch.autograd.Function):
         return _backward(ctx, do, dlse)
 
 
+def _block_args(block_mask, eq, ek, score_func_mode):
+    if block_mask is None:
+        return eq, ek, score_func_mode
+    assert eq is None and ek is None and score_func_mode == SCORE_FUNC_MODE0_NOPE, "block_mask excludes eq / ek"
+    return block_mask, block_mask, SCORE_FUNC_MODE2_BLOCK
+
+
 def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE,
-              *, window=0, prefix=0):
-    """flash_triton.py:640-641.  Two keyword-only additions, both causal masks (0 = off, exclusive):
-    window = W: sliding window, a row sees only its last W keys up to the diagonal;
-    prefix = P: prefix-LM, the first P keys are seen by every row."""
+              *, window=0, prefix=0, block_mask=None):
+    """flash_triton.py:640-641.  Keyword-only additions (no counterpart in the reference):
+    window = W: sliding window, a row sees only its last W keys up to the diagonal (causal only);
+    prefix = P: prefix-LM, the first P keys are seen by every row (causal only, excludes window);
+    block_mask: block-sparse attention -- a bool / integer tensor [bs|1, H|1, ceil(Lq/64), ceil(Lk/64)];
+    a (row, key) pair is kept iff its 64 x 64 block is non-zero (and the causal terms hold); blocks that
+    are switched off are never visited.  Excludes eq / ek."""
+    eq, ek, score_func_mode = _block_args(block_mask, eq, ek, score_func_mode)
     return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
 
 
@@ -249,9 +272,10 @@ def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func
 # Accessors for tests and benchmarks (not part of the reference's surface).
 # ---------------------------------------------------------------------------
 def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
-                       score_func_mode=SCORE_FUNC_MODE0_NOPE, *, window=0, prefix=0):
+                       score_func_mode=SCORE_FUNC_MODE0_NOPE, *, window=0, prefix=0, block_mask=None):
     """(O, LSE) with LSE in natural-log units (-inf for rows without a kept key); differentiable
     through both results."""
+    eq, ek, score_func_mode = _block_args(block_mask, eq, ek, score_func_mode)
     return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
 
 
@@ -326,7 +350,13 @@ def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_M
     p.dtype = _cabi.FA_DTYPE_BF16
     keep = []
     with torch.cuda.device(device):
-        if score_func_mode != SCORE_FUNC_MODE0_NOPE:
+        if score_func_mode == SCORE_FUNC_MODE2_BLOCK:   # eq: the block map [B|1, H|1, ceil(M/64), ceil(N/64)]
+            nbr, nbc = -(-M // _cabi.FA_MASK_BLOCK), -(-N // _cabi.FA_MASK_BLOCK)
+            bm = maybe_contiguous((eq != 0).to(torch.uint8).to(device)).expand(B, H, nbr, nbc)
+            p.eq = bm.data_ptr()
+            _set3(p.eq_stride, bm)
+            keep += [bm]
+        elif score_func_mode != SCORE_FUNC_MODE0_NOPE:
             eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
             if eq.dtype != ek.dtype:
                 eq, ek = eq.to(torch.int64), ek.to(torch.int64)

@@ -29,6 +29,7 @@ class Workload:
     ek: Optional[np.ndarray] = None   # [B, Lk] int32
     window: int = 0       # sliding window (causal only; 0 = off)
     prefix: int = 0       # prefix-LM (causal only; 0 = off)
+    block: Optional[np.ndarray] = None   # [B, ceil(Lq/64), ceil(Lk/64)] bool: block mask shared by all heads (excludes eq / ek)
 
 
 def _pack_docs(rng, L, draw_len):
@@ -80,6 +81,11 @@ def make_workload(name: str, seed: int = 0) -> Workload:
         ek = np.broadcast_to(ek, (B, Lk)).copy()
         eq = np.stack([_globalise(rng, ek[b, -Lq:], 0.05) for b in range(B)])   # the last 4 docs
         return Workload(name, B, H, H, Lq, Lk, D, "fp16", True, True, eq, ek)
+    if name == "block25_causal_16k":    # block-sparse: the diagonal blocks and a quarter of the others, under a causal mask
+        L = 16384
+        blk = rng.random((1, L // 64, L // 64)) < 0.25
+        blk |= np.eye(L // 64, dtype=bool)[None]
+        return Workload(name, 1, 32, 32, L, L, 128, "bf16", True, False, block=blk)
     if name == "window1k_causal_16k":   # sliding window of 1024 keys over 16K tokens
         return Workload(name, 1, 32, 32, 16384, 16384, 128, "bf16", True, False, window=1024)
     if name == "fp32_causal_4k":     # the fp32 kernels at a size that fills the chip
@@ -109,6 +115,8 @@ def keep_rows(w: Workload, b: int, i0: int, i1: int) -> np.ndarray:
         e_q = w.eq[b, i0:i1].astype(np.int64)[:, None]
         e_k = w.ek[b].astype(np.int64)[None, :]
         keep &= (e_q >= 0) | (e_q == e_k)
+    if w.block is not None:
+        keep &= w.block[b][(i // 64), (j // 64)]
     return keep
 
 
@@ -217,6 +225,9 @@ def executed_wave_steps(w: Workload):
             vis = vis & (j0 <= np.maximum(gap + rmax[:, None], pfx_m1)) & (j0 + 63 >= gap + rmin[:, None] - win + 1)
         if w.doc:
             vis = vis & (g[:, None] | ((lo[:, None] <= k64_hi[None, :]) & (k64_lo[None, :] <= hi[:, None])))
+        if w.block is not None:   # a wave's 32 rows lie inside one row of blocks, a key tile is one column
+            nW = len(nv)
+            vis = vis & w.block[b][np.minimum(np.arange(nW) // 2, w.block.shape[1] - 1)][:, :nK64] & (np.arange(nW) // 2 < w.block.shape[1])[:, None]
         fwd_steps += int(vis.sum())
         # dk/dv: waves of 32 keys against query tiles of 64 (permuted order)
         k32 = pad(ek, nK32 * 32, 0).reshape(nK32, 32)
@@ -231,6 +242,9 @@ def executed_wave_steps(w: Workload):
             vis = vis & ((gap + rmax[:, None] >= n0) | (n0 <= pfx_m1)) & (gap + rmin[:, None] - win + 1 <= n0 + 31)
         if w.doc:
             vis = vis & (g[:, None] | ((lo[:, None] <= k32_hi[None, :]) & (k32_lo[None, :] <= hi[:, None])))
+        if w.block is not None:   # a query tile is one row of blocks, a wave's 32 keys lie inside one column
+            nT = len(nv)
+            vis = vis & w.block[b][np.minimum(np.arange(nT), w.block.shape[1] - 1)][:, np.arange(nK32) // 2] & (np.arange(nT) < w.block.shape[1])[:, None]
         kv_steps += int(vis.sum())
     return fwd_steps, kv_steps
 
