@@ -132,7 +132,8 @@ BLOCK_CASES = [
     # B, H, Hk, M, N, D, dtype, causal, window, density, broadcast (block map shared by batch and heads)
     (1, 2, 2, 512, 512, 128, torch.bfloat16, False, 0, 0.5, False),
     (2, 2, 2, 512, 512, 128, torch.bfloat16, True, 0, 0.5, False),
-    (1, 4, 2, 450, 700, 128, torch.float16, True, 0, 0.6, True),      # grouped, ragged, rectangular
+    (1, 4, 2, 450, 700, 128, torch.float16, True, 0, 0.6, False),     # grouped (a map per query head), ragged, rectangular
+    (2, 4, 1, 260, 260, 64, torch.bfloat16, False, 0, 0.5, True),      # grouped, one map for everything
     (1, 2, 2, 300, 300, 64, torch.bfloat16, True, 0, 0.4, False),
     (1, 2, 1, 333, 520, 64, torch.float16, False, 0, 0.3, True),
     (1, 2, 2, 200, 200, 16, torch.bfloat16, True, 0, 0.5, False),
