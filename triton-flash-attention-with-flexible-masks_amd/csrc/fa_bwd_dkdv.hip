@@ -602,9 +602,11 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   // stream is better served by the 128-key form, which reads every query tile half as often.  With
   // ids a workgroup visits about a dozen tiles at 16K tokens in documents of ~512 (64-key form 9 %
   // faster); without ids the number of tiles is known here: all of them, half on average under a
-  // causal mask, at most a window's worth under a sliding window.
+  // causal mask, at most a window's worth under a sliding window.  Under a block mask the 64-key
+  // form is one column of blocks: no wave waits at a tile that only the other column needs
+  // (diagonal + 25 % random blocks at 16K tokens: 1.81 -> 1.24 ms).
   if constexpr (D > 64) {
-    if (DOC) return launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s);
+    if (DOC || a.bmask != nullptr) return launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s);
     int tiles = (a.M + 63) / 64;
     if (CAUSAL) tiles = a.win < 0x3fffffff ? min(tiles, a.win / 64 + 3) : (tiles + 1) / 2;
     tiles *= a.G;
