@@ -302,8 +302,10 @@ def test_negative_and_large_scale():
     _run_case(1, 2, 1, 256, 2304, 64, torch.bfloat16, True, True, seed=54, sm_scale=0.3)   # split tiles + sharp softmax
 
 
-def test_graph_capture_and_replay():
-    """The five calls of a step (plan, forward, delta, dk/dv, dq) captured into one HIP graph: every
+@pytest.mark.parametrize("dq_forms_delta", [False, True])
+def test_graph_capture_and_replay(dq_forms_delta):
+    """The calls of a step (plan, forward, delta, dk/dv, dq -- or plan, forward, dq forming delta, dk/dv)
+    captured into one HIP graph: every
     replay, with new inputs copied into the captured buffers and eager work in between, must give the
     eager result bit for bit (the library allocates nothing and clears its counters with kernels)."""
     import ctypes
@@ -330,12 +332,17 @@ def test_graph_capture_and_replay():
     p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
     ref = ctypes.byref(p)
 
+    if dq_forms_delta:
+        p.flags = _cabi.FA_FLAG_DQ_DELTA
+    calls = ("fa_mask_plan", "fa_fwd", "fa_bwd_dq", "fa_bwd_dkdv") if dq_forms_delta else \
+            ("fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq")
+
     def step():
         s = _stream_ptr(dev)
-        for name in ("fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
+        for name in calls:
             _cabi.check(getattr(L, name)(ref, s), name)
 
-    print("case graph capture", flush=True)
+    print("case graph capture, dq forms delta:", dq_forms_delta, flush=True)
     step()                       # eager once: kernel attributes are set outside the capture
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
