@@ -24,7 +24,10 @@ CASES = {
     "rect_doc_causal_fp16": (1, 2, 2, 16, 48, 32, torch.float16, True, True),
     "gqa_doc_causal_bf16": (1, 4, 2, 40, 40, 64, torch.bfloat16, True, True),
     "plain_noncausal_bf16": (2, 2, 2, 24, 40, 32, torch.bfloat16, False, False),
+    # block mask (64 x 64 blocks, drawn per head): "doc" is False, the map is stored as "block"
+    "block_causal_bf16": (1, 2, 1, 150, 200, 32, torch.bfloat16, True, False),
 }
+BLOCK = {"block_causal_bf16"}
 
 
 def make(name):
@@ -45,15 +48,21 @@ def make(name):
         ek = torch.from_numpy(ekn.astype(np.int32))
         eq = ek[..., N - M:].contiguous()
         out.update(eq=eq.numpy(), ek=ek.numpy())
-    o, lse, delta, dq, dk, dv = O.attention_grads(q, k, v, do, causal, None, eq, ek, 1 if doc else 0)
+    mode = 1 if doc else 0
+    if name in BLOCK:
+        bm = rng.random((B, H, -(-M // 64), -(-N // 64))) < 0.6
+        bm[:, 0, 1, :] = False   # a row of blocks without any key
+        eq, mode = torch.from_numpy(bm), 2
+        out.update(block=bm)
+    o, lse, delta, dq, dk, dv = O.attention_grads(q, k, v, do, causal, None, eq, ek, mode)
     keep = np.broadcast_to(O.keep_mask(M, N, causal, None if eq is None else eq.numpy(),
-                                       None if ek is None else ek.numpy(), 1 if doc else 0), (B, H, M, N))
+                                       None if ek is None else ek.numpy(), mode), (B, H, M, N))
     out.update(o=o.numpy(), lse=lse.numpy(), delta=delta.numpy(), dq=dq.numpy(), dk=dk.numpy(), dv=dv.numpy(),
                keep=np.packbits(keep, axis=-1), keep_shape=np.array(keep.shape))
     np.savez_compressed(Path(__file__).parent / f"{name}.npz", **out)
 
 
 if __name__ == "__main__":
-    for n in CASES:
+    for n in (sys.argv[1:] or CASES):
         make(n)
         print("wrote", n)

@@ -27,12 +27,16 @@ def test_fixture_matches_oracle_routes(path):
     eq = torch.from_numpy(d["eq"]) if doc else None
     ek = torch.from_numpy(d["ek"]) if doc else None
     M, N = q.shape[2], k.shape[2]
-    keep = np.broadcast_to(O.keep_mask(M, N, causal, d.get("eq"), d.get("ek"), int(doc)), d["keep"].shape)
+    mode = int(doc)
+    if "block" in d:   # block mask: the map travels in the place of eq
+        eq, mode = torch.from_numpy(d["block"]), 2
+        d["eq"] = d["block"]
+    keep = np.broadcast_to(O.keep_mask(M, N, causal, d.get("eq"), d.get("ek"), mode), d["keep"].shape)
     assert np.array_equal(keep, d["keep"])
-    o, lse, dq, dk, dv = O.attention_autograd(q, k, v, do, causal, None, eq, ek, int(doc), dtype=torch.float64)
+    o, lse, dq, dk, dv = O.attention_autograd(q, k, v, do, causal, None, eq, ek, mode, dtype=torch.float64)
     for name, got in (("o", o), ("lse", lse), ("dq", dq), ("dk", dk), ("dv", dv)):
         assert np.allclose(got.numpy(), d[name], atol=1e-10), name
-    if k.shape[1] == q.shape[1] or True:
+    if "block" not in d:   # the tiled restatement knows the reference's two score modes
         Ot, L2, dQ, dK, dV = O.attention_tiled(d["q"], d["k"], d["v"], d["do"], causal, 1 / np.sqrt(q.shape[-1]),
                                                d.get("eq"), d.get("ek"), int(doc), 8, 16)
         assert np.allclose(Ot, d["o"], atol=1e-10) and np.allclose(dK, d["dk"], atol=1e-10)

@@ -436,13 +436,18 @@ def test_golden_fixtures():
         eq = torch.from_numpy(z["eq"]).cuda() if doc else None
         ek = torch.from_numpy(z["ek"]).cuda() if doc else None
         mode = 1 if doc else 0
+        if "block" in z.files:   # block mask: the map travels in the place of eq
+            eq = ek = torch.from_numpy(z["block"]).cuda()
+            mode = 2
         B, H, M, _ = q.shape
         N = k.shape[2]
         keep = np.unpackbits(z["keep"], axis=-1, count=N).astype(bool)
         assert np.array_equal(mask_dump(B, H, M, N, causal, eq, ek, mode).cpu().numpy(), keep)
         out, lse = attention_with_lse(q, k, v, causal, None, eq, ek, mode)
         assert (out.float().cpu().numpy() - z["o"]).__abs__().max() <= TOL_O
-        assert np.abs(lse.cpu().numpy() - z["lse"]).max() <= TOL_LSE
+        dead = np.isinf(z["lse"])                      # rows without any kept key: -inf on both sides
+        assert np.array_equal(np.isinf(lse.cpu().numpy()), dead)
+        assert np.abs(np.where(dead, 0.0, lse.cpu().numpy() - np.where(dead, 0.0, z["lse"]))).max() <= TOL_LSE
         q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
         attention(q, k, v, causal, None, eq, ek, mode).backward(do)
         for name, got in (("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
