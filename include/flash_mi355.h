@@ -55,7 +55,7 @@ extern "C" {
    extension point): `eq` points to bytes [B, H, ceil(M/64), ceil(N/64)], eq_stride = its batch, head
    and row strides in bytes (0 allowed for batch and head), the column stride is 1; `ek`, `id_dtype`
    and the workspace are not used and fa_mask_plan is not needed.  A pair (i, j) is kept iff the byte of
-   block (i / 64, j / 64) is non-zero and the causal / window / prefix terms hold.  bf16 / fp16 only. */
+   block (i / 64, j / 64) is non-zero and the causal / window / prefix terms hold. */
 #define FA_SCORE_MODE2_BLOCK 2
 #define FA_MASK_BLOCK 64
 

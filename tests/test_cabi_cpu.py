@@ -73,12 +73,12 @@ def test_validate_codes():
     p = _good_params(buf); p.flags = 2; assert v(p) == -7
     p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; assert v(p) == 0 and v(p, 1) == 0
     p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p, 1) == -10
-    # block mask: eq carries the byte map, no workspace, no ek; not for fp32; rows of the map at least ceil(N/64) apart
+    # block mask: eq carries the byte map, no workspace, no ek; rows of the map at least ceil(N/64) apart
     p = _good_params(buf); p.score_mode = _cabi.FA_SCORE_MODE2_BLOCK; assert v(p) == -7
     p = _good_params(buf); p.score_mode = _cabi.FA_SCORE_MODE2_BLOCK; p.eq = p.q; p.eq_stride[2] = (p.N + 63) // 64
     assert v(p) == 0 and L.fa_workspace_bytes(ctypes.byref(p)) == 0
     p.eq_stride[2] -= 1; assert v(p) == -6
-    p.eq_stride[2] += 1; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p) == -10
+    p.eq_stride[2] += 1; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p) == 0
     # sliding window / prefix: causal only, not both, not negative
     p = _good_params(buf); p.window = 64; assert v(p) == 0
     p = _good_params(buf); p.prefix = 64; assert v(p) == 0

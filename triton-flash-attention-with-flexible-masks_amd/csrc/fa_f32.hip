@@ -180,11 +180,25 @@ void fwd_f32_kernel(const KArgs a) {
     wg_reduce3(g_lo, g_hi, g_glob);
     ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
   }
+  // block mask: the byte rows of the workgroup's two 64-row halves (the second one may lie past the last row)
+  const unsigned char* bm0 = nullptr;
+  const unsigned char* bm1 = nullptr;
+  if (!DOC && a.bmask != nullptr) {
+    const unsigned char* base = a.bmask + b * a.bm_bs + h * a.bm_hs;
+    bm0 = base + int64_t(2 * tile) * a.bm_rs;
+    if (2 * tile + 1 < a.nBr) bm1 = base + int64_t(2 * tile + 1) * a.bm_rs;
+  }
   auto next_kt = [&](int kt) {
     if (DOC)
       while (kt < nkt) {
         const IdSummary ks = ksum[(kt * kRows) / kSumRows];
         if (doc_may_keep(g_lo, g_hi, g_glob, ks.lo, ks.hi)) break;
+        ++kt;
+      }
+    if (!DOC && bm0 != nullptr)
+      while (kt < nkt) {   // tiles whose block is off for both halves are not even loaded
+        const int col = (kt * kRows) / FA_MASK_BLOCK;
+        if ((bm0[col] | (bm1 != nullptr ? bm1[col] : 0)) != 0) break;
         ++kt;
       }
     return kt;
@@ -211,6 +225,10 @@ void fwd_f32_kernel(const KArgs a) {
     }
     kt = kt_next;
     bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
+    if (!DOC && bm0 != nullptr && !skip) {   // the wave's 32 rows and the tile's 32 keys lie inside one block
+      const unsigned char* r = wave >= 2 ? bm1 : bm0;
+      skip = r == nullptr || r[n0 / FA_MASK_BLOCK] == 0;
+    }
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
       const int id = lid[lq];
@@ -338,11 +356,25 @@ void dq_f32_kernel(const KArgs a) {
     wg_reduce3(g_lo, g_hi, g_glob);
     ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
   }
+  // block mask: the byte rows of the workgroup's two 64-row halves (the second one may lie past the last row)
+  const unsigned char* bm0 = nullptr;
+  const unsigned char* bm1 = nullptr;
+  if (!DOC && a.bmask != nullptr) {
+    const unsigned char* base = a.bmask + b * a.bm_bs + h * a.bm_hs;
+    bm0 = base + int64_t(2 * tile) * a.bm_rs;
+    if (2 * tile + 1 < a.nBr) bm1 = base + int64_t(2 * tile + 1) * a.bm_rs;
+  }
   auto next_kt = [&](int kt) {
     if (DOC)
       while (kt < nkt) {
         const IdSummary ks = ksum[(kt * kRows) / kSumRows];
         if (doc_may_keep(g_lo, g_hi, g_glob, ks.lo, ks.hi)) break;
+        ++kt;
+      }
+    if (!DOC && bm0 != nullptr)
+      while (kt < nkt) {   // tiles whose block is off for both halves are not even loaded
+        const int col = (kt * kRows) / FA_MASK_BLOCK;
+        if ((bm0[col] | (bm1 != nullptr ? bm1[col] : 0)) != 0) break;
         ++kt;
       }
     return kt;
@@ -369,6 +401,10 @@ void dq_f32_kernel(const KArgs a) {
     }
     kt = kt_next;
     bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
+    if (!DOC && bm0 != nullptr && !skip) {   // the wave's 32 rows and the tile's 32 keys lie inside one block
+      const unsigned char* r = wave >= 2 ? bm1 : bm0;
+      skip = r == nullptr || r[n0 / FA_MASK_BLOCK] == 0;
+    }
     if (DOC && !skip) {
       const bool kv = n0 + lq < a.N;
       const int id = lid[lq];
@@ -485,11 +521,20 @@ void dkdv_f32_kernel(const KArgs a) {
       wg_reduce3(gk_lo, gk_hi, gk_unused);
       rsum = a.ksum + b * a.ks_bs + h * a.ks_hs;
     }
+    // block mask: the one or two byte columns of the workgroup's 128 keys
+    const unsigned char* bmc = (!DOC && a.bmask != nullptr) ? a.bmask + b * a.bm_bs + h * a.bm_hs + n0 / FA_MASK_BLOCK : nullptr;
+    const bool bm_two = n0 / FA_MASK_BLOCK + 1 < a.nBc;
     auto next_mt = [&](int mt) {
       if (DOC && rsum != nullptr)
         while (mt < nMt) {
           const IdSummary qs = rsum[(mt * kRows) / kSumRows];   // ids of 64 rows: any id >= 0 is a global row
           if (doc_may_keep(qs.lo, qs.hi, qs.hi >= 0, gk_lo, gk_hi)) break;
+          ++mt;
+        }
+      if (bmc != nullptr)
+        while (mt < nMt) {   // tiles whose block is off for both key columns are not even loaded
+          const unsigned char* r = bmc + int64_t((mt * kRows) / FA_MASK_BLOCK) * a.bm_rs;
+          if ((r[0] | (bm_two ? r[1] : 0)) != 0) break;
           ++mt;
         }
       return mt;
@@ -518,6 +563,8 @@ void dkdv_f32_kernel(const KArgs a) {
       mt = mt_next;
       bool skip = nw >= a.N || (CAUSAL && ((a.gap + min(m0 + kRows - 1, a.M - 1) < nw && nw > a.pfx_m1) ||
                                            a.gap + m0 - a.win + 1 > nw + 31));
+      if (bmc != nullptr && !skip)   // the wave's 32 keys and the tile's 32 rows lie inside one block
+        skip = bmc[int64_t(m0 / FA_MASK_BLOCK) * a.bm_rs + (wave >= 2 ? 1 : 0)] == 0;
       if (DOC && !skip) {
         const bool rv_ = m0 + lq < a.M;
         const int id = leq[lq];

@@ -144,7 +144,6 @@ class _Impl:
             "q, k, v must share one of torch.bfloat16 / torch.float16 / torch.float32"
         assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
         if score_func_mode == SCORE_FUNC_MODE2_BLOCK:
-            assert q.dtype != torch.float32, "block masks are implemented for bfloat16 / float16"
             nbr, nbc = -(-M // _cabi.FA_MASK_BLOCK), -(-N // _cabi.FA_MASK_BLOCK)
             assert eq.dim() == 4 and eq.shape[0] in (1, B) and eq.shape[1] in (1, H) and tuple(eq.shape[2:]) == (nbr, nbc), \
                 f"block_mask must be [bs|1, H|1, {nbr}, {nbc}] (blocks of 64 x 64)"
