@@ -106,11 +106,12 @@ def test_workspace_size():
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want   # 4 key tiles of 64: no key range is ever split
     assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want   # ... so all of it is plan
     # from 32 key tiles on, scratch for split global-row tiles: arrival counters, (max, sum) pairs, fp32
-    # partial tiles; chunks = clamp(key tiles / 32, 2, 4), splittable tiles = clamp(128 MiB / footprint, 8, 64)
+    # partial tiles; chunks = clamp(key tiles / 32, 2, 4) (finer when the launch is short of workgroups),
+    # splittable tiles = clamp(128 MiB / footprint, 8, 64), at most ceil(M / 128) + 1
     p.N = 2048
     p.ek_stride[0], p.ek_stride[1] = 4 * 2048, 2048
-    chunks, tiles = 2, 64   # 32 key tiles -> 2 chunks
-    assert (128 << 20) // (1 * 4 * chunks * 128 * (p.D + 2) * 4) >= 64
+    chunks, tiles = 2, 2   # 32 key tiles -> 2 chunks of 16; M = 128 rows -> 2 tiles
+    assert p.M == 128 and (128 << 20) // (1 * 4 * chunks * 128 * (p.D + 2) * 4) >= 64
     want = (r256(128 * 4) + r256(4 * 2048 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
             + r256(4 * 32 * 32)
             + r256(4 * tiles * 4) + r256(4 * tiles * chunks * 128 * 2 * 4) + r256(4 * tiles * chunks * 128 * p.D * 4))

@@ -205,6 +205,16 @@ def test_long_key_ranges_of_global_rows():
     _run_case(2, 2, 2, 2048, 2048, 16, torch.bfloat16, True, True, seed=24)
 
 
+def test_short_query_long_key_without_ids():
+    """Few query rows against a long key range and no ids: the operator hands the call to the kernels as
+    all-global rows, whose key range is cut into chunks for separate workgroups (up to 16 here)."""
+    from flash_mi355 import api
+    assert api._short_query_long_key(1, 2, 100, 8300, torch.bfloat16) and not api._short_query_long_key(1, 2, 100, 8300, torch.float32)
+    _run_case(1, 2, 1, 100, 8300, 128, torch.bfloat16, True, False, seed=61)
+    _run_case(1, 4, 2, 1, 9000, 64, torch.float16, False, False, seed=62)
+    _run_case(2, 2, 2, 300, 16500, 32, torch.bfloat16, True, False, seed=63, window=5000)
+
+
 def test_transposed_views_and_strided_gradients():
     """q, k, v, dO given as [B, L, H, D] storage viewed as [B, H, L, D] (cf. testing.py:59-66): the kernels
     take element strides, nothing is copied on the way in."""

@@ -146,7 +146,7 @@ static KArgs make_args(const fa_params* p) {
     a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
     a.qk_same = (p->eq == p->ek && p->M == p->N && p->eq_stride[0] == p->ek_stride[0] && p->eq_stride[1] == p->ek_stride[1] &&
                  p->eq_stride[2] == p->ek_stride[2]) ? 1 : 0;
-    const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
+    const SplitCfg sc = split_config(p->B, p->H, p->M, p->N, p->D);
     a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);
     a.sk_ml = reinterpret_cast<float*>(ws + w.off_sk_ml);

@@ -49,21 +49,34 @@ constexpr int kPermAlign = 256;
 // by different workgroups; each writes an fp32 partial result and the last one to arrive (an atomic
 // counter per tile) merges them.  The merge order is fixed, results stay reproducible.
 constexpr int kSplitMinTiles = 16;   // key tiles (of 64) per chunk below which splitting does not pay
-constexpr int kSplitKMax = 4;        // more chunks did not pay on any measured shape
+constexpr int kSplitKMax = 4;        // more chunks did not pay on any shape with enough query tiles to fill the chip
+constexpr int kSplitKMaxFew = 16;    // ... but they do when the whole launch is short of workgroups (few query rows)
 struct SplitCfg {
   int k;      // chunks per tile (1: nothing is ever split)
   int tiles;  // global-row tiles per (batch, head) that can be split
 };
 // Chunks of at least 32 key tiles (2 .. kSplitKMax of them), and as many splittable tiles as 128 MB of
 // scratch allow (8 .. 64): long sequences with few heads have many global-row tiles, each of them long.
-inline SplitCfg split_config(int B, int H, int N, int D) {
+// With so few query rows that even kSplitKMax chunks per tile leave the chip short of workgroups
+// (decoding, the tail of a long prompt) the chunks go down to kSplitMinTiles key tiles, up to
+// kSplitKMaxFew of them.  Never more splittable tiles than M rows can fill.
+inline SplitCfg split_config(int B, int H, int M, int N, int D) {
   SplitCfg c = {1, 0};
   const int nKs = (N + kSumRows - 1) / kSumRows;
   if (nKs < 2 * kSplitMinTiles) return c;   // no key range can be long enough to be cut
-  c.k = nKs / 32 < 2 ? 2 : (nKs / 32 > kSplitKMax ? kSplitKMax : nKs / 32);
+  const int qtiles = (M + 127) / 128 + 1;   // 128-row tiles of global rows a (batch, head) can have
+  const uint64_t wgs = uint64_t(B) * H * qtiles;
+  if (wgs * kSplitKMax < 512) {
+    const int kmax = int(512 / wgs) < kSplitKMaxFew ? (int(512 / wgs) > kSplitKMax ? int(512 / wgs) : kSplitKMax) : kSplitKMaxFew;
+    const int want = nKs / kSplitMinTiles;
+    c.k = want < 2 ? 2 : (want > kmax ? kmax : want);
+  } else {
+    c.k = nKs / 32 < 2 ? 2 : (nKs / 32 > kSplitKMax ? kSplitKMax : nKs / 32);
+  }
   const uint64_t per_tile = uint64_t(c.k) * 128 * (D + 2) * 4;
   const uint64_t t = (uint64_t(128) << 20) / (uint64_t(B) * H * per_tile);
   c.tiles = t < 8 ? 8 : (t > 64 ? 64 : int(t));
+  if (c.tiles > qtiles) c.tiles = qtiles;
   return c;
 }
 
@@ -285,7 +298,7 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
   // scratch of the split tiles: only when a key range can be long enough to be cut
-  const SplitCfg sc = split_config(p->B, p->H, p->N, p->D);
+  const SplitCfg sc = split_config(p->B, p->H, p->M, p->N, p->D);
   const uint64_t nsk = uint64_t(p->B) * p->H * sc.tiles;
   w.off_sk_cnt = take(nsk * 4);
   w.plan_bytes = o;      // the counters (zeroed by the plan, left at zero by every kernel) are state

@@ -111,6 +111,11 @@ def _prep_ids(e, name):
     return e
 
 
+def _short_query_long_key(B, H, M, N, dtype):
+    """No ids, fewer query tiles than half the chip has CUs, and a key range long enough to be cut (16-bit types)."""
+    return dtype != torch.float32 and B * H * ((M + 127) // 128) <= 128 and N >= 8192
+
+
 class _Impl:
     """Forward and backward shared by the two autograd functions below."""
 
@@ -157,6 +162,14 @@ class _Impl:
             assert tuple(ek.shape) == (B, H, N), "ek must be [bs, H, Lk]"
         else:
             eq = ek = None
+            if _short_query_long_key(B, H, M, N, q.dtype):
+                # Few query tiles against a long key range (decoding, the tail of a long prompt): a launch of
+                # B*H*ceil(M/128) workgroups leaves most of the chip idle while each walks every key.  Rows whose
+                # id is >= 0 see every key (flash_triton.py:114), and the kernels cut the key range of such rows
+                # into chunks that separate workgroups process and merge: the same mask, more parallelism.
+                eq = torch.zeros((B, 1, M), dtype=torch.int32, device=q.device).expand(B, H, M)
+                ek = torch.zeros((B, 1, N), dtype=torch.int32, device=q.device).expand(B, H, N)
+                score_func_mode = SCORE_FUNC_MODE1_DOC
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
 
         L = _cabi.lib()
