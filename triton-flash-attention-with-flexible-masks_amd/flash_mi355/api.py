@@ -167,8 +167,8 @@ class _Impl:
                 # B*H*ceil(M/128) workgroups leaves most of the chip idle while each walks every key.  Rows whose
                 # id is >= 0 see every key (flash_triton.py:114), and the kernels cut the key range of such rows
                 # into chunks that separate workgroups process and merge: the same mask, more parallelism.
-                eq = torch.zeros((B, 1, M), dtype=torch.int32, device=q.device).expand(B, H, M)
-                ek = torch.zeros((B, 1, N), dtype=torch.int32, device=q.device).expand(B, H, N)
+                zero = torch.zeros((1, 1, 1), dtype=torch.int32, device=q.device)   # every stride 0: one id for all
+                eq, ek = zero.expand(B, H, M), zero.expand(B, H, N)
                 score_func_mode = SCORE_FUNC_MODE1_DOC
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
 
