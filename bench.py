@@ -108,13 +108,9 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=20, warm=5):
     stream = _stream_ptr(dev)
     ref = ctypes.byref(p)
     out = {}
-    # the launches of the operator's backward: dq forms delta itself for the 16-bit types (as api.py asks
-    # for), fp32 keeps the separate delta launch
-    if w.dtype == "fp32":
-        names = [("fa_fwd", L.fa_fwd), ("fa_bwd_delta", L.fa_bwd_delta), ("fa_bwd_dkdv", L.fa_bwd_dkdv), ("fa_bwd_dq", L.fa_bwd_dq)]
-    else:
-        p.flags = _cabi.FA_FLAG_DQ_DELTA
-        names = [("fa_fwd", L.fa_fwd), ("fa_bwd_dq", L.fa_bwd_dq), ("fa_bwd_dkdv", L.fa_bwd_dkdv)]
+    # the launches of the operator's backward: dq forms delta itself, then dk/dv (as api.py asks for)
+    p.flags = _cabi.FA_FLAG_DQ_DELTA
+    names = [("fa_fwd", L.fa_fwd), ("fa_bwd_dq", L.fa_bwd_dq), ("fa_bwd_dkdv", L.fa_bwd_dkdv)]
     if w.doc:
         names.insert(0, ("fa_mask_plan", L.fa_mask_plan))
     quant = {}

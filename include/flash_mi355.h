@@ -83,7 +83,7 @@ extern "C" {
 #define FA_FLAG_DQ_DELTA 1  /* fa_bwd_dq computes delta = rowsum(o * dout) of its own rows itself (o must be set)
                                and also stores it to p->delta: the fa_bwd_delta launch is then not needed, and
                                fa_bwd_dkdv, which reads delta, goes after fa_bwd_dq on the stream.
-                               16-bit dtypes only (FA_ERR_NOT_IMPLEMENTED for fp32).  Ignored by every other call. */
+                               Ignored by every other call. */
 
 typedef struct fa_params {
   /* forward operands */

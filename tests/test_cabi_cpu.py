@@ -72,7 +72,7 @@ def test_validate_codes():
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
     p = _good_params(buf); p.flags = 2; assert v(p) == -7
     p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; assert v(p) == 0 and v(p, 1) == 0
-    p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p, 1) == -10
+    p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p, 1) == 0
     # block mask: eq carries the byte map, no workspace, no ek; rows of the map at least ceil(N/64) apart
     p = _good_params(buf); p.score_mode = _cabi.FA_SCORE_MODE2_BLOCK; assert v(p) == -7
     p = _good_params(buf); p.score_mode = _cabi.FA_SCORE_MODE2_BLOCK; p.eq = p.q; p.eq_stride[2] = (p.N + 63) // 64

@@ -378,7 +378,8 @@ def test_graph_capture_and_replay(dq_forms_delta):
 
 
 @pytest.mark.parametrize("M,D,doc,dtype", [(2304, 64, True, torch.bfloat16), (450, 128, False, torch.float16),
-                                           (1000, 128, True, torch.bfloat16), (333, 16, True, torch.float16)])
+                                           (1000, 128, True, torch.bfloat16), (333, 16, True, torch.float16),
+                                           (450, 64, True, torch.float32), (300, 128, False, torch.float32)])
 def test_dq_computes_delta(M, D, doc, dtype):
     """FA_FLAG_DQ_DELTA: fa_bwd_dq forms delta itself and leaves it for fa_bwd_dkdv; delta, dq, dk, dv
     must agree with the three-launch sequence (delta is a sum of the same products in another order:
@@ -419,7 +420,7 @@ def test_dq_computes_delta(M, D, doc, dtype):
     for name, got, w_ in zip(("dq", "dk", "dv"), (dq, dk, dv), want[1:]):
         assert not torch.isnan(got).any(), name
         err = (got.float() - w_.float()).abs().max().item()
-        assert err <= 2.0 ** -7 * max(1.0, w_.float().abs().max().item()), (name, err)
+        assert err <= (1e-4 if dtype == torch.float32 else 2.0 ** -7) * max(1.0, w_.float().abs().max().item()), (name, err)
 
 
 def test_harness_cell_runs_and_agrees():

@@ -56,7 +56,6 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->eq_stride[0] < 0 || p->eq_stride[1] < 0 || p->eq_stride[2] < (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK) return FA_ERR_STRIDE;
   }
   if ((p->flags & ~FA_FLAG_DQ_DELTA) != 0) return FA_ERR_MODE;
-  if ((p->flags & FA_FLAG_DQ_DELTA) != 0 && p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
   if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {

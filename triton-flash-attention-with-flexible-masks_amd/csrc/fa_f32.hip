@@ -321,7 +321,17 @@ void dq_f32_kernel(const KArgs a) {
   for (int s = 0; s < KS2; ++s) { qreg[s] = qp[2 * s + g]; doreg[s] = dop[2 * s + g]; }
   float L_i = a.lse[(int64_t(b) * a.H + h) * a.M + rowc];
   if (L_i == -INFINITY) L_i = INFINITY;   // row without any kept key: P = exp2(-inf) = 0
-  const float delta_i = a.delta[(int64_t(b) * a.H + h) * a.M + rowc];
+  float delta_i;
+  if (a.dq_delta) {   // delta = rowsum(O * dO) formed here (the lane and its partner hold the two halves of the row) and left for dk/dv
+    const float* op = reinterpret_cast<const float*>(a.o) + b * a.o_bs + h * a.o_hs + int64_t(rowc) * a.o_rs;
+    float part = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS2; ++s) part += op[2 * s + g] * doreg[s];
+    delta_i = xhalf_sum(part);
+    if (row < a.M && g == 0) a.delta[(int64_t(b) * a.H + h) * a.M + row] = delta_i;
+  } else {
+    delta_i = a.delta[(int64_t(b) * a.H + h) * a.M + rowc];
+  }
   const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
   const bool glob_i = eq_i >= 0;
   const int lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;

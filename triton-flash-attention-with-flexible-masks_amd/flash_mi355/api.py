@@ -214,7 +214,7 @@ class _Impl:
             _set4(p.o_stride, o); _set4(p.do_stride, do)
             _set4(p.dq_stride, dq); _set4(p.dk_stride, dk); _set4(p.dv_stride, dv)
             stream = _stream_ptr(q.device)
-            if dlse is None and q.dtype != torch.float32:
+            if dlse is None:
                 # two launches instead of the reference's three (flash_triton.py:585-634): the dq kernel
                 # forms delta = rowsum(O * dO) from rows it holds anyway and leaves it for the dk/dv kernel
                 p.flags = _cabi.FA_FLAG_DQ_DELTA
