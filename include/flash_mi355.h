@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 4
+#define FA_ABI_VERSION 5
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
@@ -84,6 +84,15 @@ extern "C" {
                                and also stores it to p->delta: the fa_bwd_delta launch is then not needed, and
                                fa_bwd_dkdv, which reads delta, goes after fa_bwd_dq on the stream.
                                Ignored by every other call. */
+#define FA_FLAG_DEBUG_NO_PAIR_WAIT 0x100
+                            /* Diagnostic, for tests of the failure path below; never set it in production.
+                               In fa_bwd_dkdv at D = 128 two waves share each block of 32 keys: one publishes P in
+                               on-chip memory, the other polls a sequence number for it.  The poll is bounded (about
+                               a millisecond) so that every wave ends whatever happens; a wave whose wait expired
+                               has used a P it cannot trust and REPORTS it by writing NaN into its 32 rows of dk
+                               (dv is not affected).  A NaN in dk after a backward with finite inputs therefore
+                               means "a pair wait expired", not an arithmetic overflow.  With this flag the poll
+                               budget is zero, so the report can be provoked without hanging or faulting anything. */
 
 typedef struct fa_params {
   /* forward operands */

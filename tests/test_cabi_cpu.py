@@ -107,7 +107,7 @@ def test_workspace_size():
     assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want   # ... so all of it is plan
     # from 32 key tiles on, scratch for split global-row tiles: arrival counters, (max, sum) pairs, fp32
     # partial tiles; chunks = clamp(key tiles / 32, 2, 4) (finer when the launch is short of workgroups),
-    # splittable tiles = clamp(128 MiB / footprint, 8, 64), at most ceil(M / 128) + 1
+    # splittable tiles = min(128 MiB / footprint, 64), at most ceil(M / 128) + 1
     p.N = 2048
     p.ek_stride[0], p.ek_stride[1] = 4 * 2048, 2048
     chunks, tiles = 2, 2   # 32 key tiles -> 2 chunks of 16; M = 128 rows -> 2 tiles
@@ -141,6 +141,44 @@ def test_python_layer_asserts_like_the_reference():
         attention(q, k, k, score_func_mode=SCORE_FUNC_MODE1_DOC)                    # doc mode without ids
     with pytest.raises(AssertionError):
         attention(q, k, k)                                                          # CPU tensors: no CPU fallback
+
+
+def test_operands_on_another_device_are_refused():
+    """Ids, k, v or dO that do not live on q's device are refused with an AssertionError before any
+    pointer reaches a kernel (checked on the helper itself: no GPU is needed to compare devices)."""
+    from flash_mi355 import api
+    q = torch.zeros(1, 1, 8, 16, device="meta")
+    api._check_same_device(q, k=torch.zeros(2, device="meta"), eq=None)
+    with pytest.raises(AssertionError, match="eq is on cpu"):
+        api._check_same_device(q, eq=torch.zeros(1, 1, 8, dtype=torch.int32))
+    with pytest.raises(AssertionError, match="v is on cpu"):
+        api._check_same_device(q, k=torch.zeros(2, device="meta"), v=torch.zeros(2))
+    import inspect
+    src = inspect.getsource(api._Impl.forward) + inspect.getsource(api._Impl.backward)
+    assert src.count("_check_same_device(q, ") >= 3   # k/v, eq/ek in forward; dO in backward
+
+
+def test_split_scratch_stays_inside_its_budget():
+    """The scratch of the split key ranges is bounded whatever the batch: with many (batch, head) pairs
+    fewer tiles per pair are splittable, down to none."""
+    L = _cabi.lib()
+    buf = ctypes.create_string_buffer(4096)
+    budget = 128 << 20
+    for (B, H, Lseq, D) in [(64, 32, 2048, 128), (32, 32, 4096, 128), (8, 32, 8192, 128), (1, 32, 16384, 128),
+                            (4, 8, 65536, 64), (256, 64, 2048, 16), (1, 4, 131072, 128)]:
+        p = _good_params(buf)
+        p.B, p.H, p.Hk, p.M, p.N, p.D = B, H, H, Lseq, Lseq, D
+        p.score_mode = 1
+        p.eq_stride[0], p.eq_stride[1], p.eq_stride[2] = Lseq, 0, 1
+        p.ek_stride[0], p.ek_stride[1], p.ek_stride[2] = Lseq, 0, 1
+        total = L.fa_workspace_bytes(ctypes.byref(p))
+        plan = L.fa_workspace_plan_bytes(ctypes.byref(p))
+        assert 0 < plan <= total and total - plan <= budget + 512, (B, H, Lseq, D, total - plan)
+    # the headline shape still splits its global-row tiles
+    p = _good_params(buf)
+    p.B, p.H, p.Hk, p.M, p.N, p.D, p.score_mode = 1, 32, 32, 16384, 16384, 128, 1
+    p.eq_stride[2] = p.ek_stride[2] = 1
+    assert L.fa_workspace_bytes(ctypes.byref(p)) - L.fa_workspace_plan_bytes(ctypes.byref(p)) > (32 << 20)
 
 
 def test_drop_in_module_name():

@@ -12,6 +12,8 @@ import numpy as np
 import pytest
 import torch
 
+from tests._tol import check_close
+
 pytestmark = pytest.mark.gpu
 
 TOL_O = 2e-2
@@ -111,5 +113,56 @@ def test_slices_against_the_oracle(name, slices):
         assert (got_l[~dead] - rl[~dead]).abs().max().item() <= TOL_LSE
         assert (out.detach()[sl].float().cpu() - ro).abs().max().item() <= TOL_O
         for nm, got, ref in (("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
-            err = (got[sl].float().cpu() - ref).abs().max().item()
-            assert err <= TOL_O * max(1.0, ref.abs().max().item() / 4), (name, b, h, nm, err)
+            check_close(f"{name} slice ({b},{h}) {nm}", got[sl], ref)
+
+
+def test_cfg2_plain_every_head_against_the_oracle():
+    """The plain configuration (no mask, not causal, D = 64, bf16) at its full size, every one of its
+    64 (batch, head) slices against the oracle, a few heads at a time (scores are 16 MB per head)."""
+    from flash_mi355 import attention_with_lse, workloads as W
+    from oracle import attention_oracle as O
+    w = W.make_workload("cfg2_plain")
+    assert (w.B, w.H, w.Lq, w.Lk, w.D, w.dtype, w.causal, w.doc) == (4, 16, 2048, 2048, 64, "bf16", False, False)
+    g = torch.Generator().manual_seed(2)
+    q, k, v, do = (torch.randn(w.B, w.H, w.Lq, w.D, generator=g).to(torch.bfloat16) for _ in range(4))
+    print("case cfg2_plain full size", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out, lse = attention_with_lse(qd, kd, vd, False, None)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    o, l = out.detach().float().cpu(), lse.detach().cpu()
+    dq, dk, dv = (t.grad.float().cpu() for t in (qd, kd, vd))
+    worst = {}
+    for b in range(w.B):
+        for h0 in range(0, w.H, 4):
+            sl = (slice(b, b + 1), slice(h0, h0 + 4))
+            ro, rl, rdq, rdk, rdv = O.attention_autograd(q[sl], k[sl], v[sl], do[sl], False, None, None, None, 0)
+            assert (l[sl] - rl).abs().max().item() <= TOL_LSE
+            assert (o[sl] - ro).abs().max().item() <= TOL_O
+            for nm, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+                worst[nm] = max(worst.get(nm, 0.0), check_close(f"cfg2 b{b} h{h0}..{h0 + 3} {nm}", got[sl], ref, quiet=True))
+    print("  cfg2_plain worst err/bound:", {n: round(r, 3) for n, r in worst.items()}, flush=True)
+
+
+def test_cfg1_fp32_doc_causal_in_full():
+    """The CPU-sized configuration (fp32, B=2 H=4 L=512 D=64, causal + document mask with the ids of its
+    definition: documents of 32..256 tokens, 5 % global) on the fp32 kernels, every element."""
+    from flash_mi355 import attention_with_lse, workloads as W, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    w = W.make_workload("cfg1_cpu_doc_causal")
+    assert (w.B, w.H, w.Lq, w.D, w.dtype, w.causal, w.doc) == (2, 4, 512, 64, "fp32", True, True)
+    g = torch.Generator().manual_seed(3)
+    q, k, v, do = (torch.randn(w.B, w.H, w.Lq, w.D, generator=g) for _ in range(4))
+    eq = torch.from_numpy(w.eq)[:, None, :].expand(w.B, w.H, w.Lq)
+    print("case cfg1_cpu_doc_causal full size", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out, lse = attention_with_lse(qd, kd, vd, True, None, eq.cuda(), eq.cuda(), SCORE_FUNC_MODE1_DOC)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    ro, rl, rdq, rdk, rdv = O.attention_autograd(q, k, v, do, True, None, eq, eq, 1)
+    tol = 2e-4   # fp32 products and accumulation throughout
+    assert not torch.isinf(rl).any()
+    assert (lse.detach().cpu() - rl).abs().max().item() <= tol
+    for nm, got, ref in (("o", out, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        err = (got.detach().float().cpu() - ref).abs().max().item()
+        assert err <= tol * max(1.0, ref.abs().max().item()), (nm, err)

@@ -55,7 +55,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->eq == nullptr) return FA_ERR_MODE;
     if (p->eq_stride[0] < 0 || p->eq_stride[1] < 0 || p->eq_stride[2] < (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK) return FA_ERR_STRIDE;
   }
-  if ((p->flags & ~FA_FLAG_DQ_DELTA) != 0) return FA_ERR_MODE;
+  if ((p->flags & ~(FA_FLAG_DQ_DELTA | FA_FLAG_DEBUG_NO_PAIR_WAIT)) != 0) return FA_ERR_MODE;
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
   if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
@@ -120,6 +120,7 @@ static KArgs make_args(const fa_params* p) {
   a.nQs = a.nKs = a.Pp = 0;
   a.qk_same = 0;
   a.dq_delta = (p->flags & FA_FLAG_DQ_DELTA) != 0;
+  a.pair_spin = (p->flags & FA_FLAG_DEBUG_NO_PAIR_WAIT) ? 0 : kPairSpinDefault;
   a.bmask = nullptr; a.bm_bs = a.bm_hs = a.bm_rs = 0;
   a.nBr = (p->M + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK; a.nBc = (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK;
   if (p->score_mode == FA_SCORE_MODE2_BLOCK) {

@@ -237,22 +237,23 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
 template <bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(256) void mask_dump_kernel(const KArgs a, uint8_t* __restrict__ out) {
   const int j = blockIdx.x * 256 + threadIdx.x;
-  const int i = blockIdx.y;
-  const int bh = blockIdx.z, b = bh / a.H, h = bh % a.H;
   if (j >= a.N) return;
-  int eq_i = 0, ek_j = 0;
-  if (DOC) {
-    eq_i = a.eq32[b * a.eq_bs + h * a.eq_hs + i];
-    ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + j];
+  // rows and (batch, head) pairs are walked with the grid's stride: grid dimensions y and z stop at 65535
+  for (int bh = blockIdx.z; bh < a.B * a.H; bh += gridDim.z) {
+    const int b = bh / a.H, h = bh % a.H;
+    const int ek_j = DOC ? a.ek32[b * a.ek_bs + h * a.ek_hs + j] : 0;
+    for (int i = blockIdx.y; i < a.M; i += gridDim.y) {
+      const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + i] : 0;
+      bool keep = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1);
+      if (!DOC && a.bmask != nullptr)
+        keep = keep && a.bmask[b * a.bm_bs + h * a.bm_hs + int64_t(i / FA_MASK_BLOCK) * a.bm_rs + j / FA_MASK_BLOCK] != 0;
+      out[(int64_t(bh) * a.M + i) * a.N + j] = keep ? 1 : 0;
+    }
   }
-  bool keep = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1);
-  if (!DOC && a.bmask != nullptr)
-    keep = keep && a.bmask[b * a.bm_bs + h * a.bm_hs + int64_t(i / FA_MASK_BLOCK) * a.bm_rs + j / FA_MASK_BLOCK] != 0;
-  out[(int64_t(bh) * a.M + i) * a.N + j] = keep ? 1 : 0;
 }
 
 int launch_mask_dump(const KArgs& a, bool causal, bool doc, uint8_t* out, hipStream_t s) {
-  dim3 grid((a.N + 255) / 256, a.M, a.B * a.H);
+  dim3 grid((a.N + 255) / 256, a.M < 65535 ? a.M : 65535, a.B * a.H < 65535 ? a.B * a.H : 65535);
   if (causal && doc) hipLaunchKernelGGL((mask_dump_kernel<true, true>), grid, dim3(256), 0, s, a, out);
   else if (causal) hipLaunchKernelGGL((mask_dump_kernel<true, false>), grid, dim3(256), 0, s, a, out);
   else if (doc) hipLaunchKernelGGL((mask_dump_kernel<false, true>), grid, dim3(256), 0, s, a, out);

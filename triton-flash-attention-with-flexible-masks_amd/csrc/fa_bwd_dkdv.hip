@@ -21,14 +21,13 @@
 // are visited.  The query heads of a grouped-query group are walked inside the kernel, so dK, dV
 // are written once, already summed (the reference sums afterwards, flash_triton.py:635-637).
 #include "fa_tile.h"
-#ifndef FA_KV_PRE
-#define FA_KV_PRE 4
-#endif
-#ifndef FA_KV_PRE2
-#define FA_KV_PRE2 3
-#endif
 
 namespace fa {
+
+// Operand fragments requested ahead of the MFMA that consumes them, in program order (measured
+// optimum of a sweep over 2..6): row-wise reads of the first products, transposed reads of the second.
+constexpr int kKvPre = 4;
+constexpr int kKvPre2 = 3;
 
 // SPLIT = true : two waves per block of 32 keys, NKB key blocks per workgroup, roles split over the
 //                wave pairs as described above (D = 128: one wave cannot hold both operand sets and
@@ -51,7 +50,11 @@ void bwd_dkdv_kernel(const KArgs a) {
   constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][NKB key blocks][2 x 1024]: P in the element type
   constexpr int P_BYTES = 2048;
   constexpr int FLAG_OFF = P_OFF + 2 * NKB * P_BYTES;   // [2 (block parity)][NKB] sequence numbers of the published P
-  constexpr int kPairSpinMax = 1 << 14;   // ~1 ms: orders of magnitude above a legitimate wait
+  // Polls of the pair flag before the gradient wave gives up (kPairSpinDefault, about a millisecond:
+  // orders of magnitude above a legitimate wait; 0 with FA_FLAG_DEBUG_NO_PAIR_WAIT).  A wave that
+  // gave up has used a P it cannot trust: it says so by writing NaN into its dK rows at the end.
+  const int pair_spin_max = a.pair_spin;
+  int pair_lost = 0;
   constexpr int NW = SPLIT ? 2 * NKB : NKB;
   static_assert(NW >= 4, "the four auxiliary arrays of a tile are loaded by waves 0..3");
   using Loader = TileLoader<DL, BQ, D, NW>;
@@ -250,7 +253,7 @@ void bwd_dkdv_kernel(const KArgs a) {
         x = E::mfma32(ra, frag[ks], x);
       }
       {
-        constexpr int PRE = KS < FA_KV_PRE ? KS : FA_KV_PRE;
+        constexpr int PRE = KS < kKvPre ? KS : kKvPre;
         __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
         for (int i = 0; i < KS - PRE; ++i) {
@@ -265,7 +268,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     auto second_product = [&](const char* tr, const vec8 (&yf)[2], const int qb) __attribute__((always_inline)) {
       // NM transposed fragments (two LDS reads each), requested PRE fragments ahead of their MFMA
       // in program order
-      constexpr int NM = 2 * DBN, PRE = NM < FA_KV_PRE2 ? NM : FA_KV_PRE2;
+      constexpr int NM = 2 * DBN, PRE = NM < kKvPre2 ? NM : kKvPre2;
       auto fetch = [&](const int i) __attribute__((always_inline)) {
         const int half = i / DBN, db = i % DBN;
         const int goff = (2 * qb + half) * 16 * DL * 2;
@@ -329,7 +332,12 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) dl[q4] = *reinterpret_cast<const f32x4*>(aux + 256 + (32 * qb + 8 * q4 + 4 * g) * 4);
       const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
-      for (int spin = 0; spin < kPairSpinMax && __builtin_amdgcn_readfirstlane(lds_flag_load(fl)) != pair_seq; ++spin) __builtin_amdgcn_s_sleep(1);
+      bool arrived = false;
+      for (int spin = 0; spin <= pair_spin_max; ++spin) {
+        if (__builtin_amdgcn_readfirstlane(lds_flag_load(fl)) == pair_seq) { arrived = true; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (!arrived) pair_lost = 1;
       vec8 pr8[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const vec8*>(pbuf + half * 1024);
@@ -373,7 +381,7 @@ void bwd_dkdv_kernel(const KArgs a) {
         dp = E::mfma32(ro, frag2[ks], dp);
       }
       {
-        constexpr int NM = 2 * KS, PRE = NM < FA_KV_PRE ? NM : FA_KV_PRE;
+        constexpr int NM = 2 * KS, PRE = NM < kKvPre ? NM : kKvPre;
         __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
         for (int i = 0; i < NM - PRE; ++i) {
@@ -403,7 +411,7 @@ void bwd_dkdv_kernel(const KArgs a) {
       // requested PRE MFMAs ahead in program order, P and dS are converted just in time; the
       // scheduling barriers pin that order.
       {
-        constexpr int NM = 4 * DBN, PRE = NM < FA_KV_PRE2 + 1 ? NM : FA_KV_PRE2 + 1;
+        constexpr int NM = 4 * DBN, PRE = NM < kKvPre2 + 1 ? NM : kKvPre2 + 1;
         auto fetch = [&](const int i) __attribute__((always_inline)) {
           const int half = i / (2 * DBN), db = (i % (2 * DBN)) / 2;
           const char* t = (i & 1) ? lqt : ldo;
@@ -571,6 +579,12 @@ void bwd_dkdv_kernel(const KArgs a) {
         }
     };
     if (SPLIT) {
+      if (role == 1 && pair_lost) {   // the bounded wait expired somewhere: this wave's dK is not to be trusted
+#pragma unroll
+        for (int db = 0; db < DBN; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[db][r] = __builtin_nanf("");
+      }
       store(role == 0 ? dvrow : dkrow, acc, role == 0 ? 1.0f : a.scale);
     } else {
       store(dvrow, acc, 1.0f);
@@ -579,9 +593,8 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
 }
 
-#ifndef FA_KV_SHORT_TILES
-#define FA_KV_SHORT_TILES 32
-#endif
+// Query tiles per workgroup (no ids) below which the 64-key role-split form is launched.
+constexpr int kKvShortTiles = 32;
 template <typename Tag, int D, bool CAUSAL, bool DOC, int NKB>
 static int launch_nkb(const KArgs& a, hipStream_t s) {
   constexpr bool SPLIT = D > 64;
@@ -610,7 +623,7 @@ static int launch_one(const KArgs& a, hipStream_t s) {
     int tiles = (a.M + 63) / 64;
     if (CAUSAL) tiles = a.win < 0x3fffffff ? min(tiles, a.win / 64 + 3) : (tiles + 1) / 2;
     tiles *= a.G;
-    return tiles < FA_KV_SHORT_TILES ? launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s) : launch_nkb<Tag, D, CAUSAL, DOC, 4>(a, s);
+    return tiles < kKvShortTiles ? launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s) : launch_nkb<Tag, D, CAUSAL, DOC, 4>(a, s);
   } else {
     return launch_nkb<Tag, D, CAUSAL, DOC, 4>(a, s);
   }

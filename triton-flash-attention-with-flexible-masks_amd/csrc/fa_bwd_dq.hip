@@ -10,14 +10,13 @@
 // Same workgroup shape, LDS staging and tile skipping as the forward kernel.
 
 #include "fa_tile.h"
-#ifndef FA_DQ_PRE
-#define FA_DQ_PRE 4
-#endif
-#ifndef FA_DQ_PRE2
-#define FA_DQ_PRE2 3
-#endif
 
 namespace fa {
+
+// Operand fragments requested ahead of the MFMA that consumes them, in program order (measured
+// optimum of a sweep over 2..6): row-wise K / V reads, transposed K reads of the dQ product.
+constexpr int kDqPre = 4;
+constexpr int kDqPre2 = 3;
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 3 : 2, D <= 64 ? 3 : 2)))
@@ -137,7 +136,7 @@ void bwd_dq_kernel(const KArgs a) {
         dp = E::mfma32(vf, dof[ks], dp);
       }
       {
-        constexpr int NM = 2 * KS, PRE = NM < FA_DQ_PRE ? NM : FA_DQ_PRE;
+        constexpr int NM = 2 * KS, PRE = NM < kDqPre ? NM : kDqPre;
         __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
         for (int i = 0; i < NM - PRE; ++i) {
@@ -165,7 +164,7 @@ void bwd_dq_kernel(const KArgs a) {
       // program order, dS is converted just in time; the scheduling barriers pin that order (left
       // to itself the scheduler puts every read right before its MFMA).
       {
-        constexpr int NM = 2 * DBN, PRE = NM < FA_DQ_PRE2 ? NM : FA_DQ_PRE2;
+        constexpr int NM = 2 * DBN, PRE = NM < kDqPre2 ? NM : kDqPre2;
         auto fetch = [&](const int i) __attribute__((always_inline)) {
           const int half = i / DBN, db = i % DBN;
           const int goff = (2 * kb + half) * 16 * DL * 2;

@@ -55,11 +55,15 @@ struct SplitCfg {
   int k;      // chunks per tile (1: nothing is ever split)
   int tiles;  // global-row tiles per (batch, head) that can be split
 };
-// Chunks of at least 32 key tiles (2 .. kSplitKMax of them), and as many splittable tiles as 128 MB of
-// scratch allow (8 .. 64): long sequences with few heads have many global-row tiles, each of them long.
+// Chunks of at least 32 key tiles (2 .. kSplitKMax of them), and as many splittable tiles as the
+// scratch budget allows (at most 64): long sequences with few heads have many global-row tiles, each
+// of them long.  The budget is a hard bound on the scratch part of the workspace: with many (batch,
+// head) pairs it buys fewer tiles per pair, down to none (such launches have workgroups to spare and
+// short key ranges per tile; with fewer than two tiles in the budget at 4 chunks, 2 chunks are tried).
 // With so few query rows that even kSplitKMax chunks per tile leave the chip short of workgroups
 // (decoding, the tail of a long prompt) the chunks go down to kSplitMinTiles key tiles, up to
 // kSplitKMaxFew of them.  Never more splittable tiles than M rows can fill.
+constexpr uint64_t kSplitScratchBudget = uint64_t(128) << 20;   // bytes of sk_ml + sk_o
 inline SplitCfg split_config(int B, int H, int M, int N, int D) {
   SplitCfg c = {1, 0};
   const int nKs = (N + kSumRows - 1) / kSumRows;
@@ -73,12 +77,19 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D) {
   } else {
     c.k = nKs / 32 < 2 ? 2 : (nKs / 32 > kSplitKMax ? kSplitKMax : nKs / 32);
   }
-  const uint64_t per_tile = uint64_t(c.k) * 128 * (D + 2) * 4;
-  const uint64_t t = (uint64_t(128) << 20) / (uint64_t(B) * H * per_tile);
-  c.tiles = t < 8 ? 8 : (t > 64 ? 64 : int(t));
+  auto tiles_for = [&](int k) {
+    const uint64_t per_tile = uint64_t(k) * 128 * (D + 2) * 4;
+    const uint64_t t = kSplitScratchBudget / (uint64_t(B) * H * per_tile);
+    return t > 64 ? 64 : int(t);
+  };
+  c.tiles = tiles_for(c.k);
+  if (c.tiles < 2 && c.k > 2) { c.k = 2; c.tiles = tiles_for(2); }
   if (c.tiles > qtiles) c.tiles = qtiles;
+  if (c.tiles <= 0) { c.tiles = 0; c.k = 1; }
   return c;
 }
+
+constexpr int kPairSpinDefault = 1 << 14;
 
 struct bf16_t {};
 struct fp16_t {};
@@ -256,6 +267,7 @@ struct KArgs {
   int Pp;                 // entries of the permuted order per (b, h)
   int nQs, nKs;           // summary entries per (b, h)
   int dq_delta;           // the dq kernel computes delta from O and dO itself and stores it
+  int pair_spin;          // dk/dv, role-split form: polls of the pair flag before the gradient wave gives up
   // block mask (FA_SCORE_MODE2_BLOCK): bytes [B, H, nBr, nBc] per 64 x 64 block of (row, key) pairs, or null
   const unsigned char* bmask;
   int64_t bm_bs, bm_hs, bm_rs;

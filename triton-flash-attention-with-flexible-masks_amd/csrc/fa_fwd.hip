@@ -12,9 +12,10 @@
 //   O^T += V^T P^T : A = V^T via ds_read_b64_tr_b16, B = P^T taken straight from
 //                  the S^T accumulators (the key order of the accumulator
 //                  registers is absorbed into the V^T read pattern).
-//   The softmax reference point of a row is only moved (and O, l rescaled) when the
-//   row maximum has grown by more than 2^8 since it was last set, so most tiles
-//   skip the rescale; the result is mathematically unchanged.
+//   The softmax reference point of a row is only moved (and O, l rescaled) when a lane's
+//   partial row sum of a tile, taken against the reference point as it stands, exceeds 2^12
+//   (or the point is not set yet), so most tiles skip both the row maximum and the
+//   rescale; the result is mathematically unchanged.
 // Tiles of keys that cannot hold a kept element for the 128 rows (by the id
 // summaries of the mask plan) are never loaded; per wave, tiles that are fully
 // masked for its 32 rows are skipped and tiles that are fully kept take a path
@@ -22,14 +23,12 @@
 
 #include "fa_tile.h"
 
-#ifndef FA_FWD_PRE
-#define FA_FWD_PRE 4
-#endif
-#ifndef FA_FWD_PRE2
-#define FA_FWD_PRE2 4
-#endif
-
 namespace fa {
+
+// Operand fragments requested ahead of the MFMA that consumes them, in program order (measured
+// optimum of a sweep over 2..8): K rows of the first product, transposed V reads of the second.
+constexpr int kFwdPre = 4;
+constexpr int kFwdPre2 = 4;
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 3 : 2, D <= 64 ? 3 : 2)))
@@ -145,7 +144,7 @@ void fwd_kernel(const KArgs a) {
     // Instruction order of this region: keep several K fragments in flight ahead of the MFMA that
     // consumes them (an LDS read takes about as long as three MFMAs).
     {
-      constexpr int NQK = 2 * KS, PRE = NQK < FA_FWD_PRE ? NQK : FA_FWD_PRE;
+      constexpr int NQK = 2 * KS, PRE = NQK < kFwdPre ? NQK : kFwdPre;
       __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
       for (int i = 0; i < NQK - PRE; ++i) {
@@ -223,7 +222,7 @@ void fwd_kernel(const KArgs a) {
     // PRE MFMAs ahead in program order, P is converted just in time; the scheduling barriers pin
     // that order (left to itself the scheduler puts every read right before its MFMA).
     {
-      constexpr int NPV = 4 * DBN, PRE = NPV < FA_FWD_PRE2 ? NPV : FA_FWD_PRE2;
+      constexpr int NPV = 4 * DBN, PRE = NPV < kFwdPre2 ? NPV : kFwdPre2;
       auto fetch = [&](const int i) __attribute__((always_inline)) {
         const int c16 = i / DBN, db = i % DBN;
         return lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * DL * 2, lv + lo.tr[db][1] + c16 * 16 * DL * 2);

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libflash_mi355.so"
 
-FA_ABI_VERSION = 4
+FA_ABI_VERSION = 5
 FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
 FA_SCORE_MODE2_BLOCK = 2
@@ -22,6 +22,7 @@ FA_DTYPE_FP32 = 2
 FA_IDTYPE_I32 = 0
 FA_IDTYPE_I64 = 1
 FA_FLAG_DQ_DELTA = 1
+FA_FLAG_DEBUG_NO_PAIR_WAIT = 0x100
 
 # every symbol include/flash_mi355.h declares
 EXPORTS = (

@@ -111,6 +111,13 @@ def _prep_ids(e, name):
     return e
 
 
+def _check_same_device(ref, **others):
+    """Every tensor whose address is handed to a kernel lives on the device the kernels run on (a host
+    or foreign pointer would be a memory fault on the GPU, not an error)."""
+    for name, t in others.items():
+        assert t is None or t.device == ref.device, f"{name} is on {t.device}, q is on {ref.device}: all operands must share q's device"
+
+
 def _short_query_long_key(B, H, M, N, dtype):
     """No ids, fewer query tiles than half the chip has CUs, and a key range long enough to be cut (16-bit types)."""
     return dtype != torch.float32 and B * H * ((M + 127) // 128) <= 128 and N >= 8192
@@ -145,6 +152,9 @@ class _Impl:
         assert window >= 0 and prefix >= 0 and not (window and prefix), "window and prefix exclude each other"
         assert causal or not (window or prefix), "window / prefix are causal masks"
         assert q.is_cuda and k.is_cuda and v.is_cuda, "flash_mi355 runs on the GPU only"
+        _check_same_device(q, k=k, v=v)
+        if score_func_mode != SCORE_FUNC_MODE2_BLOCK:   # (a block map is moved to q's device below)
+            _check_same_device(q, eq=eq, ek=ek)
         assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, \
             "q, k, v must share one of torch.bfloat16 / torch.float16 / torch.float32"
         assert k.shape[0] == B and v.shape[0] == B and v.shape[2] == N
@@ -198,6 +208,7 @@ class _Impl:
         if do is None:   # only LSE was used
             do = torch.zeros_like(o)
         do = _aligned(maybe_contiguous(do))
+        _check_same_device(q, do=do, dlse=dlse)
         with torch.cuda.device(q.device):
             plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix)
             p = plan.p
@@ -369,7 +380,7 @@ def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_M
             _set3(p.eq_stride, bm)
             keep += [bm]
         elif score_func_mode != SCORE_FUNC_MODE0_NOPE:
-            eq, ek = _prep_ids(eq, "eq"), _prep_ids(ek, "ek")
+            eq, ek = _prep_ids(eq, "eq").to(device), _prep_ids(ek, "ek").to(device)
             if eq.dtype != ek.dtype:
                 eq, ek = eq.to(torch.int64), ek.to(torch.int64)
             p.eq, p.ek = eq.data_ptr(), ek.data_ptr()

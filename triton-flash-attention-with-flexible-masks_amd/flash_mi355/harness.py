@@ -124,7 +124,7 @@ def run_attn(func_names: Sequence[str], shape: Sequence[int], is_causal: bool, d
              check_times: int = 3, bench_times: int = 50, warmup_times: int = 10, device: str = "cuda"):
     """One (shape, causal, dtype) cell of the matrix; returns (check records, bench records)."""
     impls = implementations()
-    tdt = {"fp16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    tdt = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[dtype]   # testing.py:158
     shape = list(shape)
     checks, benches = [], []
     if check_times > 0:
