@@ -132,8 +132,16 @@ def attention_closed_form(q, k, v, causal=False, sm_scale=None, eq=None, ek=None
 
 
 def attention_grads(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
-                    score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float64, window=0, prefix=0):
-    """Explicit-formula (O, LSE, delta, dQ, dK, dV); dK, dV reduced over the GQA group."""
+                    score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float64, window=0, prefix=0, store_dtype=None):
+    """Explicit-formula (O, LSE, delta, dQ, dK, dV); dK, dV reduced over the GQA group.
+
+    store_dtype (torch.bfloat16 / torch.float16, default None = exact): round where the reference's
+    kernels round to the tensors' element type -- P before P V and P^T dO (flash_triton.py:126,291),
+    O as it is stored and read back for delta (:539,165), dS before dS K and dS^T Q (:306,417).
+    Everything else stays in ``dtype``.  Shows what error those storage roundings alone put into the
+    gradients (an implementation that follows the reference cannot be closer to the exact gradients
+    than this); with store_dtype=None the exact formulas are evaluated."""
+    rnd = (lambda x: x) if store_dtype is None else (lambda x: x.to(store_dtype).to(dtype))
     B, H, Lq, D = q.shape
     Hk, Lk = k.shape[1], k.shape[2]
     if sm_scale is None:
@@ -149,10 +157,12 @@ def attention_grads(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
         s = torch.matmul(qf, kf.transpose(-1, -2)) * sm_scale
         lse0 = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)
         p = torch.where(keep, torch.exp(s - lse0[..., None]), torch.zeros((), dtype=dtype))
+        if store_dtype is not None:
+            o = rnd(torch.matmul(rnd(p), vf))                       # :126, stored :539
         delta = (o * dof).sum(-1)                                   # flash_triton.py:165
-        dv = torch.matmul(p.transpose(-1, -2), dof)                 # :291
+        dv = torch.matmul(rnd(p).transpose(-1, -2), dof)            # :291
         dp = torch.matmul(dof, vf.transpose(-1, -2))                # :299
-        ds = p * (dp - delta[..., None])                            # :301
+        ds = rnd(p * (dp - delta[..., None]))                       # :301,306
         dq = torch.matmul(ds, kf) * sm_scale                        # :420,425
         dk = torch.matmul(ds.transpose(-1, -2), qf) * sm_scale      # :308,313
         if Hk != H:                                                 # :635-637

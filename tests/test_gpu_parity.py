@@ -80,8 +80,14 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
     for name, got, ref in (("dq", qd.grad, ref_dq), ("dk", kd.grad, ref_dk), ("dv", vd.grad, ref_dv)):
         assert got.shape == ref.shape, name
         assert not torch.isnan(got).any(), name
-        # per element: 2e-2 where |ref| <= 4, one bf16 ulp of the reference value above (tests/_tol.py)
-        check_close(name, got, ref, tol_o)
+        # per element: 2e-2 where |ref| <= 4, one bf16 ulp of the reference value above (tests/_tol.py).
+        # The bound is stated for N(0,1) inputs at the default scale D^-0.5.  A caller-given scale s times
+        # the default sharpens the softmax, and the error that the 16-bit storage of O puts into delta (the
+        # reference forms delta from the stored O too, flash_triton.py:165) reaches dQ and dK multiplied by
+        # sm_scale: such stress cases get 2e-2 * s (tests/test_oracle.py::
+        # test_storage_rounding_sets_the_gradient_error_floor shows the floor on the CPU).
+        sharp = 1.0 if sm_scale is None else max(1.0, abs(sm_scale) * math.sqrt(D))
+        check_close(name, got, ref, tol_o * sharp)
 
 
 CASES = [
