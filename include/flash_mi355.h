@@ -174,6 +174,22 @@ int fa_mask_plan(const fa_params* p, void* stream);
 /* O = softmax(q k^T * sm_scale + mask) v ; lse = log2-sum-exp2 of the scaled scores. */
 int fa_fwd(const fa_params* p, void* stream);
 
+/* fa_fwd for callers that cannot allocate device memory and hold no workspace (code under HIP graph
+   capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+   Same operands and results as fa_mask_plan + fa_fwd, but p->workspace / p->workspace_bytes are
+   ignored: the mask plan and the scratch of the split key ranges live in a static device array of
+   FA_STATIC_WS_BYTES inside the library (held by every GPU the library runs on until the process
+   ends).  The call enqueues the plan kernels and the forward on `stream` and allocates nothing, on
+   the host or the device.  Problems whose plan does not fit the array are refused with
+   FA_ERR_WORKSPACE (the plan needs about 12 bytes per query row and 5 per key, times the batch, times
+   the heads unless the ids' head stride is 0; the headline shape B=1 H=32 L=16384 takes 0.4 MB plus
+   split scratch).  Every call on a GPU uses that GPU's one array, which keeps the last call's
+   contents: calls that overlap on one GPU (different streams, different threads) race and must be
+   ordered by the caller; a backward needs its own fa_mask_plan into a caller's workspace.
+   With score_mode 0 or 2 there is no workspace and the call is fa_fwd. */
+#define FA_STATIC_WS_BYTES (32u << 20)
+int fa_fwd_static(const fa_params* p, void* stream);
+
 /* delta = rowsum(o * dout). */
 int fa_bwd_delta(const fa_params* p, void* stream);
 

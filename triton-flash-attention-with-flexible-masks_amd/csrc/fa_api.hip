@@ -1,6 +1,8 @@
 // C ABI of the library (see include/flash_mi355.h): argument validation that
 // mirrors the asserts of FlashAttention.forward (flash_triton.py:508-530),
 // translation of fa_params into the kernel-side view, and dispatch.
+#include <atomic>
+
 #include "fa_common.h"
 
 using namespace fa;
@@ -94,7 +96,7 @@ extern "C" uint64_t fa_workspace_plan_bytes(const fa_params* p) {
   return ws_layout(p).plan_bytes;
 }
 
-static KArgs make_args(const fa_params* p) {
+static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratchBudget) {
   KArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;
   a.dout = p->dout; a.dq = p->dq; a.dk = p->dk; a.dv = p->dv; a.delta = p->delta;
@@ -128,7 +130,7 @@ static KArgs make_args(const fa_params* p) {
     a.bm_bs = p->eq_stride[0]; a.bm_hs = p->eq_stride[1]; a.bm_rs = p->eq_stride[2];
   }
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
-    const WsLayout w = ws_layout(p);
+    const WsLayout w = ws_layout(p, split_budget);
     char* ws = reinterpret_cast<char*>(p->workspace);
     a.eq32 = reinterpret_cast<const int*>(ws + w.off_eq32);
     a.ek32 = reinterpret_cast<const int*>(ws + w.off_ek32);
@@ -146,7 +148,7 @@ static KArgs make_args(const fa_params* p) {
     a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
     a.qk_same = (p->eq == p->ek && p->M == p->N && p->eq_stride[0] == p->ek_stride[0] && p->eq_stride[1] == p->ek_stride[1] &&
                  p->eq_stride[2] == p->ek_stride[2]) ? 1 : 0;
-    const SplitCfg sc = split_config(p->B, p->H, p->M, p->N, p->D);
+    const SplitCfg sc = w.split;
     a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);
     a.sk_ml = reinterpret_cast<float*>(ws + w.off_sk_ml);
@@ -176,6 +178,56 @@ extern "C" int fa_fwd(const fa_params* p, void* stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (p->dtype == FA_DTYPE_FP32) return finish(launch_fwd_f32(make_args(p), p->D, causal, doc, s));
   return finish(launch_fwd(make_args(p), p->dtype, p->D, causal, doc, s));
+}
+
+// ---------------------------------------------------------------------------
+// Forward without any allocation anywhere: the mask plan and the scratch of the split key ranges
+// live in a static device array instead of a caller's workspace.  Every GPU the library runs on
+// holds its own copy of the array at its own address until the process ends; the address is looked
+// up once per device (with that device current) and only that pointer is ever handed to kernels,
+// memsets or copies -- the array's name is a host-side stand-in, not a device address.
+// ---------------------------------------------------------------------------
+constexpr uint64_t kStaticSplitBudget = uint64_t(24) << 20;   // of FA_STATIC_WS_BYTES; the rest is for the plan
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_WS_BYTES];
+static std::atomic<void*> g_scratch_ptr[64];
+
+static int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // this device's copy (the current device)
+    if (e != hipSuccess) return (int)e;
+    if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // racing first calls find the same address
+  }
+  *out = ptr;
+  return 0;
+}
+
+extern "C" int fa_fwd_static(const fa_params* p, void* stream) {
+  if (p == nullptr) return FA_ERR_NULLPTR;
+  if (p->score_mode != FA_SCORE_MODE1_DOC) return fa_fwd(p, stream);   // no workspace in these modes
+  fa_params q = *p;
+  q.workspace = reinterpret_cast<void*>(uintptr_t(256));   // placeholder for the checks below; replaced before any launch
+  q.workspace_bytes = ~uint64_t(0);
+  int rc = fa_validate(&q, 0);
+  if (rc != FA_OK) return rc;
+  const WsLayout w = ws_layout(&q, kStaticSplitBudget);
+  if (w.total > FA_STATIC_WS_BYTES) return FA_ERR_WORKSPACE;   // sizes beyond the static array
+  void* ws = nullptr;
+  if (int e = static_scratch(&ws)) return finish(e);
+  q.workspace = ws;
+  q.workspace_bytes = FA_STATIC_WS_BYTES;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // the plan rewrites everything the kernels read (ids, order, summaries) and zeroes the arrival
+  // counters with a kernel, so nothing of an earlier call's contents is ever looked at
+  if (int e = launch_mask_plan(&q, w, s)) return finish(e);
+  const bool causal = q.causal != 0;
+  if (q.dtype == FA_DTYPE_FP32) return finish(launch_fwd_f32(make_args(&q, kStaticSplitBudget), q.D, causal, true, s));
+  return finish(launch_fwd(make_args(&q, kStaticSplitBudget), q.dtype, q.D, causal, true, s));
 }
 
 extern "C" int fa_bwd_delta(const fa_params* p, void* stream) {

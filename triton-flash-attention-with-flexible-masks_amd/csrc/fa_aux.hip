@@ -228,7 +228,7 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
     const int gap = p->N > p->M ? p->N - p->M : 0;
     hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
                        p->causal ? gap : -1, p->prefix > 0 ? ((p->prefix < p->N ? p->prefix : p->N) - 1) / kSumRows + 1 : 0, perm, peq, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
-                       p->B * p->H * split_config(p->B, p->H, p->M, p->N, p->D).tiles);
+                       p->B * p->H * w.split.tiles);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   return 0;

@@ -64,7 +64,7 @@ struct SplitCfg {
 // (decoding, the tail of a long prompt) the chunks go down to kSplitMinTiles key tiles, up to
 // kSplitKMaxFew of them.  Never more splittable tiles than M rows can fill.
 constexpr uint64_t kSplitScratchBudget = uint64_t(128) << 20;   // bytes of sk_ml + sk_o
-inline SplitCfg split_config(int B, int H, int M, int N, int D) {
+inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget = kSplitScratchBudget) {
   SplitCfg c = {1, 0};
   const int nKs = (N + kSumRows - 1) / kSumRows;
   if (nKs < 2 * kSplitMinTiles) return c;   // no key range can be long enough to be cut
@@ -79,7 +79,7 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D) {
   }
   auto tiles_for = [&](int k) {
     const uint64_t per_tile = uint64_t(k) * 128 * (D + 2) * 4;
-    const uint64_t t = kSplitScratchBudget / (uint64_t(B) * H * per_tile);
+    const uint64_t t = budget / (uint64_t(B) * H * per_tile);
     return t > 64 ? 64 : int(t);
   };
   c.tiles = tiles_for(c.k);
@@ -287,9 +287,11 @@ struct WsLayout {
   uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum;  // bytes
   uint64_t off_sk_cnt, off_sk_ml, off_sk_o, total;
   uint64_t plan_bytes;   // leading part that carries state from the plan to the kernels; the rest is scratch
+  SplitCfg split;        // split of long key ranges this layout has scratch for
 };
 
-inline WsLayout ws_layout(const fa_params* p) {
+// split_budget: bytes the scratch of the split key ranges (sk_ml, sk_o) may take
+inline WsLayout ws_layout(const fa_params* p, uint64_t split_budget = kSplitScratchBudget) {
   WsLayout w;
   w.Hq1 = (p->eq_stride[1] == 0) ? 1 : p->H;
   w.Hk1 = (p->ek_stride[1] == 0) ? 1 : p->H;
@@ -310,7 +312,8 @@ inline WsLayout ws_layout(const fa_params* p) {
   w.off_qsum = take(uint64_t(p->B) * w.Hq1 * w.nQs * sizeof(IdSummary));
   w.off_ksum = take(uint64_t(p->B) * w.Hk1 * w.nKs * sizeof(IdSummary));
   // scratch of the split tiles: only when a key range can be long enough to be cut
-  const SplitCfg sc = split_config(p->B, p->H, p->M, p->N, p->D);
+  const SplitCfg sc = split_config(p->B, p->H, p->M, p->N, p->D, split_budget);
+  w.split = sc;
   const uint64_t nsk = uint64_t(p->B) * p->H * sc.tiles;
   w.off_sk_cnt = take(nsk * 4);
   w.plan_bytes = o;      // the counters (zeroed by the plan, left at zero by every kernel) are state

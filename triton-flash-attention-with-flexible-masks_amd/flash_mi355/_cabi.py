@@ -23,12 +23,13 @@ FA_IDTYPE_I32 = 0
 FA_IDTYPE_I64 = 1
 FA_FLAG_DQ_DELTA = 1
 FA_FLAG_DEBUG_NO_PAIR_WAIT = 0x100
+FA_STATIC_WS_BYTES = 32 << 20
 
 # every symbol include/flash_mi355.h declares
 EXPORTS = (
     "fa_version", "fa_params_size", "fa_error_string", "fa_last_hip_error", "fa_validate",
     "fa_workspace_bytes", "fa_workspace_plan_bytes", "fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq",
-    "fa_mask_dump",
+    "fa_mask_dump", "fa_fwd_static",
 )
 
 
@@ -76,7 +77,7 @@ def lib() -> ctypes.CDLL:
     L.fa_workspace_bytes.argtypes = [POINTER(FaParams)]
     L.fa_workspace_plan_bytes.restype = c_uint64
     L.fa_workspace_plan_bytes.argtypes = [POINTER(FaParams)]
-    for name in ("fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
+    for name in ("fa_mask_plan", "fa_fwd", "fa_fwd_static", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
         fn = getattr(L, name)
         fn.restype = c_int
         fn.argtypes = [POINTER(FaParams), c_void_p]
