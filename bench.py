@@ -81,6 +81,10 @@ def parse_args():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device copies of 1 GiB: the reference point that scales "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE readings to bytes")
+    ap.add_argument("--only-headline", action="store_true", help="skip the short measurements of the other configurations")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of the benchmark: print the sustained bf16 MFMA rate of the chip (a bare MFMA loop "
+                         "with small-integer and with random operands, libfa_probe.so), four launches each")
     return ap.parse_args()
 
 
@@ -148,6 +152,38 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=20, warm=5):
     return out
 
 
+def measure_other_config(name, torch, steps=20, warmup=5):
+    """One short operator-level measurement (forward + backward per step) of another benchmark configuration,
+    same accounting as the headline line."""
+    from flash_mi355 import attention, workloads as W
+    w = W.make_workload(name)
+    q, k, v, do, eq, ek = make_inputs(w, torch)
+    mode = 1 if w.doc else (2 if w.block is not None else 0)
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        attention(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, mode, window=w.window, prefix=w.prefix).backward(do)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    kept, tiles, _ = W.count_mask(w)
+    f = W.flops(w, "fb", kept, tiles)
+    ex = W.executed_flops(w) if w.dtype != "fp32" else None   # the emulation follows the 16-bit kernels' tiling
+    out = {"dtype": w.dtype, "shape": [w.B, w.H, w.Lq, w.Lk, w.D], "causal": w.causal, "doc_mask": w.doc, "steps": steps,
+           "ms_per_step": round(ms, 4), "tflops_tile_effective": round(f["tile"] / ms * 1e-9, 1),
+           "tflops_dense_equivalent": round(f["dense"] / ms * 1e-9, 1)}
+    if ex is not None:
+        out["tflops_executed"] = round((ex["fwd"] + ex["dq"] + ex["dkdv"]) / ms * 1e-9, 1)
+        out["pct_of_mfma_peak"] = round(100 * out["tflops_executed"] / PEAK_TFLOPS[w.dtype], 2)
+    return out
+
+
 def cpu_baseline(w, heads, torch):
     """The reference's eager path (testing.py:32-47) on the host cores for `heads` (b, h) slices."""
     from oracle import attention_oracle as O
@@ -190,6 +226,22 @@ def main():
         print("bench.py measures one GPU: this operator shards over (batch, head) with no "
               "communication and this build uses a single GPU; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.mfma_probe:
+        from flash_mi355.build import PROBE_LIB_PATH
+        probe = ctypes.CDLL(str(PROBE_LIB_PATH))
+        probe.fa_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+        out = {}
+        for label, rnd in (("small_integers", 0), ("random_bf16", 1)):
+            rates = []
+            for _ in range(4):
+                tf_ = ctypes.c_float(0)
+                rc = probe.fa_probe_mfma_rate(rnd, 40000, ctypes.byref(tf_))
+                assert rc == 0, f"probe failed with hipError {rc}"
+                rates.append(round(tf_.value, 1))
+            out[label] = rates
+        print(json.dumps({"probe": "v_mfma_f32_32x32x16_bf16, 8 workgroups of 4 waves per CU, 4 accumulators per wave",
+                          "tflops": out, "datasheet_peak": PEAK_TFLOPS["bf16"]}))
+        return
     import torch
     from flash_mi355 import attention, workloads as W
 
@@ -278,6 +330,12 @@ def main():
         "pct_of_mfma_peak_tile_effective": round(100 * value / peak, 2),
         "detail": detail, "roofline": roofline,
     }
+    if not args.only_headline:
+        # the other configurations of the benchmark definition, measured in this same run
+        del q, k, v, do, eq, ek
+        torch.cuda.empty_cache()
+        names = [n for n in W.WORKLOADS if n != w.name]
+        line["other_configs"] = {n: measure_other_config(n, torch) for n in names}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w, args.cpu_heads, torch)
     print(json.dumps(line))

@@ -236,9 +236,43 @@ void bwd_dq_kernel(const KArgs a) {
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
+    // (up to four chunks of four steps are requested together: every device-scope load is a round
+    // trip of its own, so they are put in flight side by side instead of one after the other)
     constexpr int C4 = D / 4;
     const float* bo = a.sk_o + tbase * a.split_k * (128 * D);
     const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
+    auto finish_row = [&](int mrow, int c, f32x4 acc) __attribute__((always_inline)) {
+      const typename E::vec2 x0 = E::cvt2(acc[0] * a.scale, acc[1] * a.scale);
+      const typename E::vec2 x1 = E::cvt2(acc[2] * a.scale, acc[3] * a.scale);
+      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
+      *reinterpret_cast<typename E::vec4*>(dqp + int64_t(mrow) * a.dq_rs + 4 * c) = x;
+    };
+    if (nsplit <= 4) {
+      constexpr int IT = 4, NS = 4;
+      for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
+        f32x4 x[IT][NS];
+        int mrow[IT];
+#pragma unroll
+        for (int u = 0; u < IT; ++u) {
+          const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
+          mrow[u] = i < 128 * C4 ? prm[r] : -1;
+#pragma unroll
+          for (int sp = 0; sp < NS; ++sp) x[u][sp] = load_dev4(bo + min(sp, nsplit - 1) * (128 * D) + r * D + 4 * c);
+        }
+#pragma unroll
+        for (int u = 0; u < IT; ++u) {
+          if (mrow[u] < 0) continue;
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int sp = 0; sp < NS; ++sp) {   // fixed order: chunk 0 first, as the one-by-one form below
+            const float w = sp < nsplit ? 1.f : 0.f;
+            acc[0] += w * x[u][sp][0]; acc[1] += w * x[u][sp][1]; acc[2] += w * x[u][sp][2]; acc[3] += w * x[u][sp][3];
+          }
+          finish_row(mrow[u], (i0 + 256 * u) % C4, acc);
+        }
+      }
+      return;
+    }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
       const int r = i / C4, c = i % C4;
       const int mrow = prm[r];
@@ -248,10 +282,7 @@ void bwd_dq_kernel(const KArgs a) {
         const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
         acc[0] += x[0]; acc[1] += x[1]; acc[2] += x[2]; acc[3] += x[3];
       }
-      const typename E::vec2 x0 = E::cvt2(acc[0] * a.scale, acc[1] * a.scale);
-      const typename E::vec2 x1 = E::cvt2(acc[2] * a.scale, acc[3] * a.scale);
-      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
-      *reinterpret_cast<typename E::vec4*>(dqp + int64_t(mrow) * a.dq_rs + 4 * c) = x;
+      finish_row(mrow, c, acc);
     }
     return;
   }

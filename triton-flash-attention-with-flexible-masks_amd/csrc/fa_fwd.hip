@@ -294,11 +294,57 @@ void fwd_kernel(const KArgs a) {
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
-    // merge: the whole workgroup walks the tile, one float4 of one row per thread and step
+    // merge: the whole workgroup walks the tile, one float4 of one row per thread and step.  The
+    // partial results come through device-scope loads, each a round trip of its own: up to four chunks
+    // of four steps are requested together (16 + 16 loads in flight per thread) instead of one by one.
     constexpr int C4 = D / 4;
     const float* bo = a.sk_o + tbase * a.split_k * (128 * D);
     const float* bml = a.sk_ml + tbase * a.split_k * (128 * 2);
     const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
+    auto finish_row = [&](int mrow, int c, float mmax, float lsum, f32x4 acc) __attribute__((always_inline)) {
+      const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+      if (c == 0) lsep[mrow] = lsum > 0.f ? mmax + fast_log2(lsum) : -INFINITY;
+      const typename E::vec2 x0 = E::cvt2(acc[0] * inv, acc[1] * inv);
+      const typename E::vec2 x1 = E::cvt2(acc[2] * inv, acc[3] * inv);
+      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
+      *reinterpret_cast<typename E::vec4*>(op + int64_t(mrow) * a.o_rs + 4 * c) = x;
+    };
+    if (nsplit <= 4) {
+      constexpr int IT = 4, NS = 4;
+      for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
+        float m_[IT][NS], l_[IT][NS];
+        f32x4 x[IT][NS];
+        int mrow[IT];
+#pragma unroll
+        for (int u = 0; u < IT; ++u) {
+          const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
+          mrow[u] = i < 128 * C4 ? prm[r] : -1;
+#pragma unroll
+          for (int sp = 0; sp < NS; ++sp) {
+            const int spc = min(sp, nsplit - 1);   // chunks past the last one repeat it (weight 0 below)
+            load_dev(bml + spc * 256 + r * 2, m_[u][sp], l_[u][sp]);
+            x[u][sp] = load_dev4(bo + spc * (128 * D) + r * D + 4 * c);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < IT; ++u) {
+          if (mrow[u] < 0) continue;
+          float mmax = -INFINITY;
+#pragma unroll
+          for (int sp = 0; sp < NS; ++sp) mmax = fmaxf(mmax, m_[u][sp]);
+          float lsum = 0.f;
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int sp = 0; sp < NS; ++sp) {
+            const float w = (sp >= nsplit || m_[u][sp] == -INFINITY) ? 0.f : fast_exp2(m_[u][sp] - mmax);
+            lsum += w * l_[u][sp];
+            acc[0] += w * x[u][sp][0]; acc[1] += w * x[u][sp][1]; acc[2] += w * x[u][sp][2]; acc[3] += w * x[u][sp][3];
+          }
+          finish_row(mrow[u], (i0 + 256 * u) % C4, mmax, lsum, acc);
+        }
+      }
+      return;
+    }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
       const int r = i / C4, c = i % C4;
       const int mrow = prm[r];
@@ -319,12 +365,7 @@ void fwd_kernel(const KArgs a) {
         const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
         acc[0] += w * x[0]; acc[1] += w * x[1]; acc[2] += w * x[2]; acc[3] += w * x[3];
       }
-      const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-      if (c == 0) lsep[mrow] = lsum > 0.f ? mmax + fast_log2(lsum) : -INFINITY;
-      const typename E::vec2 x0 = E::cvt2(acc[0] * inv, acc[1] * inv);
-      const typename E::vec2 x1 = E::cvt2(acc[2] * inv, acc[3] * inv);
-      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
-      *reinterpret_cast<typename E::vec4*>(op + int64_t(mrow) * a.o_rs + 4 * c) = x;
+      finish_row(mrow, c, mmax, lsum, acc);
     }
     return;
   }

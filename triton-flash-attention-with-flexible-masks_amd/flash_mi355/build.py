@@ -21,6 +21,9 @@ LIB_PATH = PKG_DIR / "libflash_mi355.so"
 OBJ_DIR = PKG_DIR / "_obj"
 
 SOURCES = ["fa_api.hip", "fa_aux.hip", "fa_fwd.hip", "fa_bwd_dq.hip", "fa_bwd_dkdv.hip", "fa_f32.hip"]
+# measurement aid of bench.py --mfma-probe (sustained MFMA rate of the chip); a library of its own
+PROBE_SOURCE = "probe_mfma.hip"
+PROBE_LIB_PATH = PKG_DIR / "libfa_probe.so"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -61,6 +64,12 @@ def build(force: bool = True, verbose: bool = False, extra_flags=()) -> Path:
             lines = [l for l in log.splitlines() if "packed-fp32-ops" not in l]
             if lines:
                 print(f"--- {src.name}\n" + "\n".join(lines))
+    probe_src = CSRC / PROBE_SOURCE
+    if force or not PROBE_LIB_PATH.exists() or PROBE_LIB_PATH.stat().st_mtime < probe_src.stat().st_mtime:
+        cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", str(probe_src), "-o", str(PROBE_LIB_PATH)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {PROBE_SOURCE}:\n{r.stderr[-4000:]}")
     objs = [str(OBJ_DIR / (Path(n).stem + ".o")) for n in SOURCES]
     if jobs or not LIB_PATH.exists():
         cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *objs]
