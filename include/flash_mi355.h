@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 5
+#define FA_ABI_VERSION 6
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
@@ -71,10 +71,10 @@ extern "C" {
 #define FA_ERR_NULLPTR          -1
 #define FA_ERR_UNSUPPORTED_D    -2   /* D not in {16,32,64,128}: flash_triton.py:512 */
 #define FA_ERR_DTYPE            -3
-#define FA_ERR_SHAPE            -4   /* H % Hk != 0, causal with N < M, sizes <= 0 */
+#define FA_ERR_SHAPE            -4   /* H % Hk != 0, causal with N < M (without qpos), sizes <= 0 */
 #define FA_ERR_ALIGN            -5
 #define FA_ERR_STRIDE           -6
-#define FA_ERR_MODE             -7   /* unknown score mode, or doc mode without ids */
+#define FA_ERR_MODE             -7   /* unknown score mode, doc mode without ids, window / prefix / qpos misuse */
 #define FA_ERR_WORKSPACE        -8   /* workspace missing or too small */
 #define FA_ERR_HIP              -9   /* kernel launch failed; see fa_last_hip_error */
 #define FA_ERR_NOT_IMPLEMENTED -10
@@ -134,6 +134,17 @@ typedef struct fa_params {
                     the causal term becomes (max(0,N-M) + i >= j) || (j < prefix)                     */
   int32_t window;
   int32_t prefix;
+  /* Per-row causal positions (no counterpart in the reference, whose causal bound is the one offset
+     max(0,N-M) of flash_triton.py:521): int32 [B, M], row stride 1, or NULL.  With causal != 0 and
+     score_mode == FA_SCORE_MODE1_DOC, row i of batch b has its diagonal at key qpos[b][i] instead of
+     max(0,N-M)+i: keep needs j <= qpos[b][i] (and j > qpos[b][i] - window).  Values are clamped to
+     >= -1 (-1: the row sees no key).  This is what a packed batch needs whose query and key
+     boundaries differ (every sequence bottom-right aligned on its own: the tail of a longer key
+     sequence, chunked prefill, decoding): the ids confine a row to its sequence and qpos places its
+     diagonal.  N >= M is not required then.  Excludes prefix.  Read by fa_mask_plan only (which
+     stores the positions with the plan), and by fa_mask_dump. */
+  const int32_t* qpos;
+  int64_t qpos_stride;    /* batch stride of qpos in elements (0: one vector for every batch) */
 } fa_params;
 
 /* ABI version of the loaded library (== FA_ABI_VERSION of the header it was built from). */

@@ -55,7 +55,7 @@ LOG2E = 1.4426950408889634
 
 
 def keep_mask(Lq: int, Lk: int, causal: bool, eq=None, ek=None,
-              score_func_mode: int = SCORE_FUNC_MODE0_NOPE, window: int = 0, prefix: int = 0) -> np.ndarray:
+              score_func_mode: int = SCORE_FUNC_MODE0_NOPE, window: int = 0, prefix: int = 0, qpos=None) -> np.ndarray:
     """Boolean keep-mask, broadcastable to [B, H, Lq, Lk] (True = attend).
 
     causal: keep iff (max(0, Lk-Lq) + i) >= j     (flash_triton.py:107,521)
@@ -64,20 +64,28 @@ def keep_mask(Lq: int, Lk: int, causal: bool, eq=None, ek=None,
     as its extension point), both need causal and exclude each other:
     window > 0: sliding window, additionally j > gap + i - window (a row sees its last `window` keys)
     prefix > 0: prefix-LM, the causal term becomes (gap + i >= j) or (j < prefix)
+    qpos [B|1, Lq]: per-row causal positions (the library's; no counterpart in the reference): the
+    diagonal of row i sits at key qpos[i] instead of gap + i, i.e. the one offset of
+    flash_triton.py:521 becomes a per-row one -- what a packed batch needs when every sequence is
+    bottom-right aligned on its own.  Needs causal, excludes prefix.
     """
     assert window >= 0 and prefix >= 0 and not (window and prefix)
     assert causal or not (window or prefix)
+    assert qpos is None or (causal and not prefix)
     keep = np.ones((1, 1, Lq, Lk), dtype=bool)
     if causal:
         gap = max(0, Lk - Lq)
-        i = np.arange(Lq, dtype=np.int64)[:, None]
         j = np.arange(Lk, dtype=np.int64)[None, :]
-        c = (gap + i) >= j
+        if qpos is None:
+            pos = (gap + np.arange(Lq, dtype=np.int64))[None, :, None]            # [1, Lq, 1]
+        else:
+            pos = np.asarray(qpos).astype(np.int64).reshape(-1, Lq)[:, :, None]   # [B|1, Lq, 1]
+        c = pos >= j
         if prefix:
             c = c | (j < prefix)
         if window:
-            c = c & (j > gap + i - window)
-        keep = keep & c[None, None]
+            c = c & (j > pos - window)
+        keep = keep & c[:, None]
     if score_func_mode == SCORE_FUNC_MODE1_DOC:
         eq = np.asarray(eq).astype(np.int64)
         ek = np.asarray(ek).astype(np.int64)
@@ -107,7 +115,7 @@ def _expand_kv(x: torch.Tensor, H: int) -> torch.Tensor:
 
 def attention_closed_form(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
                           score_func_mode=SCORE_FUNC_MODE0_NOPE,
-                          dtype=torch.float32, window=0, prefix=0) -> Tuple[torch.Tensor, torch.Tensor]:
+                          dtype=torch.float32, window=0, prefix=0, qpos=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """(O, LSE) with O = softmax(q k^T * scale + mask) v, LSE natural-log.
 
     Follows testing.py:32-47 with every operand up-cast to ``dtype`` first.
@@ -122,7 +130,8 @@ def attention_closed_form(q, k, v, causal=False, sm_scale=None, eq=None, ek=None
     keep = torch.from_numpy(keep_mask(
         Lq, Lk, causal,
         None if eq is None else eq.detach().cpu().numpy(),
-        None if ek is None else ek.detach().cpu().numpy(), score_func_mode, window, prefix))
+        None if ek is None else ek.detach().cpu().numpy(), score_func_mode, window, prefix,
+        None if qpos is None else qpos.detach().cpu().numpy()))
     s = torch.where(keep, s, torch.full((), float("-inf"), dtype=dtype))
     lse = torch.logsumexp(s, dim=-1)                       # -inf on fully masked rows
     p = torch.exp(s - torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)[..., None])
@@ -132,7 +141,7 @@ def attention_closed_form(q, k, v, causal=False, sm_scale=None, eq=None, ek=None
 
 
 def attention_grads(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
-                    score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float64, window=0, prefix=0, store_dtype=None):
+                    score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float64, window=0, prefix=0, store_dtype=None, qpos=None):
     """Explicit-formula (O, LSE, delta, dQ, dK, dV); dK, dV reduced over the GQA group.
 
     store_dtype (torch.bfloat16 / torch.float16, default None = exact): round where the reference's
@@ -149,11 +158,12 @@ def attention_grads(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
     with torch.no_grad():
         qf, kf, vf = q.to(dtype), _expand_kv(k.to(dtype), H), _expand_kv(v.to(dtype), H)
         dof = do.to(dtype)
-        o, lse = attention_closed_form(q, k, v, causal, sm_scale, eq, ek, score_func_mode, dtype, window, prefix)
+        o, lse = attention_closed_form(q, k, v, causal, sm_scale, eq, ek, score_func_mode, dtype, window, prefix, qpos)
         keep = torch.from_numpy(keep_mask(
             Lq, Lk, causal,
             None if eq is None else eq.detach().cpu().numpy(),
-            None if ek is None else ek.detach().cpu().numpy(), score_func_mode, window, prefix))
+            None if ek is None else ek.detach().cpu().numpy(), score_func_mode, window, prefix,
+            None if qpos is None else qpos.detach().cpu().numpy()))
         s = torch.matmul(qf, kf.transpose(-1, -2)) * sm_scale
         lse0 = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)
         p = torch.where(keep, torch.exp(s - lse0[..., None]), torch.zeros((), dtype=dtype))
@@ -173,12 +183,12 @@ def attention_grads(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
 
 
 def attention_autograd(q, k, v, do, causal=False, sm_scale=None, eq=None, ek=None,
-                       score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float32, window=0, prefix=0):
+                       score_func_mode=SCORE_FUNC_MODE0_NOPE, dtype=torch.float32, window=0, prefix=0, qpos=None):
     """(O, LSE, dQ, dK, dV) via torch autograd through the closed form."""
     qd = q.detach().to(dtype).requires_grad_(True)
     kd = k.detach().to(dtype).requires_grad_(True)
     vd = v.detach().to(dtype).requires_grad_(True)
-    o, lse = attention_closed_form(qd, kd, vd, causal, sm_scale, eq, ek, score_func_mode, dtype, window, prefix)
+    o, lse = attention_closed_form(qd, kd, vd, causal, sm_scale, eq, ek, score_func_mode, dtype, window, prefix, qpos)
     o.backward(do.to(dtype))
     return o.detach(), lse.detach(), qd.grad, kd.grad, vd.grad
 

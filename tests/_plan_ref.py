@@ -7,8 +7,11 @@ SUM = 64
 INT_MAX, INT_MIN = 2**31 - 1, -2**31
 
 
-def plan_q(eq, M):
-    """eq: int array [M].  Returns perm [Pp], header dict, summaries list of dicts."""
+def plan_q(eq, M, pos=None):
+    """eq: int array [M]; pos: key position of every row's diagonal (default: the row index, to which
+    visits() adds the causal gap; the device plan stores gap + row, or the caller's per-row positions).
+    Returns perm [Pp], header dict, summaries list of dicts (rmin / rmax over the positions)."""
+    pos = np.arange(M) if pos is None else np.asarray(pos)
     Pp = (M + 255) // 256 * 256 + 256
     local = np.nonzero(eq < 0)[0]
     glob = np.nonzero(eq >= 0)[0]
@@ -24,8 +27,8 @@ def plan_q(eq, M):
         ids = eq[rows]
         loc = ids[ids < 0]
         sums.append(dict(lo=int(loc.min()) if len(loc) else INT_MAX, hi=int(loc.max()) if len(loc) else INT_MIN,
-                         glob=int((ids >= 0).any()), rmin=int(rows.min()) if len(rows) else INT_MAX,
-                         rmax=int(rows.max()) if len(rows) else -1, nvalid=len(rows)))
+                         glob=int((ids >= 0).any()), rmin=int(pos[rows].min()) if len(rows) else INT_MAX,
+                         rmax=int(pos[rows].max()) if len(rows) else -1, nvalid=len(rows)))
     hdr = dict(nL=nL, nG=nG, nLp=nLp, nT128=(nLp + (nG + 127) // 128 * 128) // 128)
     return perm, hdr, sums
 

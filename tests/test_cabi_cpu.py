@@ -71,6 +71,11 @@ def test_validate_codes():
     p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
     p = _good_params(buf); p.flags = 2; assert v(p) == -7
+    # per-row causal positions: only with causal + ids, not with a prefix; they lift the N >= M rule
+    p = _good_params(buf); p.qpos = p.q; assert v(p) == -7           # no ids
+    p = _good_params(buf); p.qpos = p.q; p.score_mode = 1; p.eq = p.ek = p.q; p.causal = 0; assert v(p, 2) == -7
+    p = _good_params(buf); p.qpos = p.q; p.score_mode = 1; p.eq = p.ek = p.q; p.prefix = 4; assert v(p, 2) == -7
+    p = _good_params(buf); p.qpos = p.q; p.score_mode = 1; p.eq = p.ek = p.q; p.M, p.N = 256, 128; assert v(p, 2) == -8   # past the shape check: no workspace
     p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; assert v(p) == 0 and v(p, 1) == 0
     p = _good_params(buf); p.flags = _cabi.FA_FLAG_DQ_DELTA; p.dtype = _cabi.FA_DTYPE_FP32; assert v(p, 1) == 0
     # block mask: eq carries the byte map, no workspace, no ek; rows of the map at least ceil(N/64) apart
@@ -101,7 +106,7 @@ def test_workspace_size():
     p.ek_stride[0], p.ek_stride[1], p.ek_stride[2] = 4 * 256, 256, 1   # per head
     r256 = lambda x: (x + 255) // 256 * 256
     Pp = 256 + 256
-    want = (r256(128 * 4) + r256(4 * 256 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+    want = (r256(128 * 4) + r256(4 * 256 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
             + r256(4 * 4 * 32))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want   # 4 key tiles of 64: no key range is ever split
     assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want   # ... so all of it is plan
@@ -112,7 +117,7 @@ def test_workspace_size():
     p.ek_stride[0], p.ek_stride[1] = 4 * 2048, 2048
     chunks, tiles = 2, 2   # 32 key tiles -> 2 chunks of 16; M = 128 rows -> 2 tiles
     assert p.M == 128 and (128 << 20) // (1 * 4 * chunks * 128 * (p.D + 2) * 4) >= 64
-    want = (r256(128 * 4) + r256(4 * 2048 * 4) + 2 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+    want = (r256(128 * 4) + r256(4 * 2048 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
             + r256(4 * 32 * 32)
             + r256(4 * tiles * 4) + r256(4 * tiles * chunks * 128 * 2 * 4) + r256(4 * tiles * chunks * 128 * p.D * 4))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want

@@ -30,7 +30,8 @@ def _ids(rng, B, H, L, kind):
 
 
 def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
-              id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE, window=0, prefix=0):
+              id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE, window=0, prefix=0,
+              qpos=None):
     from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
     from oracle import attention_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -48,9 +49,19 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
             ek = torch.from_numpy(ekn).to(id_dtype)
         else:
             ek = torch.from_numpy(_ids(rng, B, H, N, ids_kind)).to(id_dtype)[:, None, :].expand(B, H, N)
-        eq = ek[:, :, N - M:]  # queries are the last M positions (self-attention when M == N)
+        if N >= M:
+            eq = ek[:, :, N - M:]  # queries are the last M positions (self-attention when M == N)
+        else:                      # more queries than keys (only with per-row positions): ids of their own
+            eq = torch.from_numpy(_ids(rng, B, H, M, ids_kind)).to(id_dtype)[:, None, :].expand(B, H, M)
+    if isinstance(qpos, str):      # per-row causal positions: "random" (any order, -1 = sees nothing) or "steps" (packed sequences)
+        if qpos == "random":
+            qpos = rng.integers(-1, N + 4, (B, M))
+        else:
+            qpos = np.minimum(np.arange(M)[None] + np.cumsum(rng.random((1, M)) < 0.02, axis=1) * 37, N + 3)
+        qpos = torch.from_numpy(qpos).to(torch.int32)
     print(f"case B{B} H{H}/{Hk} M{M} N{N} D{D} {dtype} causal={causal} doc={doc} seed={seed} ids={ids_kind} "
-          f"window={window} prefix={prefix}", flush=True)
+          f"window={window} prefix={prefix} qpos={None if qpos is None else tuple(qpos.shape)}", flush=True)
+    qposd = None if qpos is None else qpos.cuda()
 
     qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
     eqd = eq.cuda() if eq is not None else None
@@ -59,10 +70,10 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
         eqd = eq[:, :1].contiguous().cuda().expand(B, H, M)
         ekd = ek[:, :1].contiguous().cuda().expand(B, H, N)
     out, lse = attention_with_lse(qd.detach(), kd.detach(), vd.detach(), causal, sm_scale, eqd, ekd, mode,
-                                  window=window, prefix=prefix)
+                                  window=window, prefix=prefix, qpos=qposd)
     torch.cuda.synchronize()
     ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, sm_scale, eq, ek, mode,
-                                                                   window=window, prefix=prefix)
+                                                                   window=window, prefix=prefix, qpos=qpos)
     # rows without any kept key: O = 0, LSE = -inf on both sides
     dead = torch.isinf(ref_lse)
     assert torch.equal(torch.isinf(lse.cpu()), dead)
@@ -73,7 +84,7 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
     assert o_err <= tol_o, f"O err {o_err}"
     if not check_bwd:
         return
-    out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode, window=window, prefix=prefix)
+    out2 = attention(qd, kd, vd, causal, sm_scale, eqd, ekd, mode, window=window, prefix=prefix, qpos=qposd)
     out2.backward(do.cuda())
     torch.cuda.synchronize()
     assert torch.equal(out2.detach(), out)
@@ -115,6 +126,41 @@ CASES = [
     c[0], c[1], c[2], c[3], c[4], c[5], str(c[6]).split(".")[-1], c[7], c[8]))
 def test_fwd_bwd_parity(case):
     _run_case(*case, seed=1234)
+
+
+QPOS_CASES = [
+    # B, H, Hk, M, N, D, dtype, window, positions, ids
+    (1, 2, 2, 300, 300, 128, torch.bfloat16, 0, "random", "uniform"),
+    (2, 2, 1, 200, 520, 64, torch.float16, 0, "random", "uniform"),
+    (1, 2, 2, 333, 77, 128, torch.bfloat16, 0, "random", "uniform"),     # more queries than keys
+    (1, 2, 2, 700, 900, 128, torch.bfloat16, 0, "steps", "uniform"),
+    (1, 2, 2, 700, 900, 64, torch.bfloat16, 40, "steps", "alllocal"),    # with a sliding window
+    (1, 1, 1, 260, 2200, 128, torch.bfloat16, 0, "random", "allglobal"), # split key ranges of global rows
+    (1, 2, 2, 130, 190, 16, torch.bfloat16, 7, "random", "uniform"),
+    (1, 2, 2, 257, 257, 32, torch.float16, 0, "steps", "uniform"),
+]
+
+
+@pytest.mark.parametrize("case", QPOS_CASES, ids=lambda c: "M%d-N%d-D%d-w%d-%s-%s" % (c[3], c[4], c[5], c[7], c[8], c[9]))
+def test_per_row_causal_positions(case):
+    """qpos: every row carries the key position of its own diagonal (arbitrary order, -1 = the row sees
+    nothing, more queries than keys allowed); forward, LSE and all gradients against the oracle."""
+    B, H, Hk, M, N, D, dtype, window, kind, ids = case
+    _run_case(B, H, Hk, M, N, D, dtype, True, True, seed=4321 + M, ids_kind=ids, window=window, qpos=kind)
+
+
+def test_per_row_positions_mask_bit_exact():
+    from flash_mi355 import mask_dump, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    rng = np.random.default_rng(11)
+    for (B, H, M, N, window) in [(2, 2, 200, 260, 0), (1, 3, 150, 90, 0), (2, 1, 129, 129, 9)]:
+        ek = torch.from_numpy(np.stack([_ids(rng, B, H, N, "uniform") for _ in range(H)], axis=1))
+        eq = torch.from_numpy(np.stack([_ids(rng, B, H, M, "uniform") for _ in range(H)], axis=1))
+        for pos in (rng.integers(-3, N + 4, (B, M)), rng.integers(-1, N, (1, M))):
+            got = mask_dump(B, H, M, N, True, eq.cuda(), ek.cuda(), SCORE_FUNC_MODE1_DOC, window=window,
+                            qpos=torch.from_numpy(pos).cuda()).cpu().numpy()
+            ref = np.broadcast_to(O.keep_mask(M, N, True, eq.numpy(), ek.numpy(), 1, window=window, qpos=np.maximum(pos, -1)), (B, H, M, N))
+            assert np.array_equal(got, ref)
 
 
 def test_mask_bit_exact():
@@ -505,6 +551,7 @@ def test_device_mask_plan_matches_host_restatement():
     o_ek = off; off += r256(B * H * Np * 4)
     o_pm = off; off += r256(B * H * Pp * 4)
     o_pq = off; off += r256(B * H * Pp * 4)
+    o_pp = off; off += r256(B * H * Pp * 4)
     off += r256(B * H * ((Mp + 1023) // 1024) * 4)     # per-chunk counts of the partition
     o_hd = off; off += r256(B * H * 16)
     o_qs = off; off += r256(B * H * nQs * 32)
@@ -514,6 +561,8 @@ def test_device_mask_plan_matches_host_restatement():
     i32 = lambda o, n: ws[o:o + 4 * n].view(np.int32)
     perm = i32(o_pm, B * H * Pp).reshape(B, H, Pp)
     peq = i32(o_pq, B * H * Pp).reshape(B, H, Pp)
+    ppos = i32(o_pp, B * H * Pp).reshape(B, H, Pp)
+    assert np.array_equal(ppos, np.where(perm >= 0, perm + (N - M), -1))   # diagonal positions: gap + row
     hdr = i32(o_hd, B * H * 4).reshape(B, H, 4)
     qs = i32(o_qs, B * H * nQs * 8).reshape(B, H, nQs, 8)
     ks = i32(o_ks, B * H * nKs * 8).reshape(B, H, nKs, 8)
@@ -528,9 +577,10 @@ def test_device_mask_plan_matches_host_restatement():
             assert list(hdr[b, h]) == [rh["nL"], rh["nG"], rh["nLp"], rh["nT128"]]
             for t, s_ in enumerate(rq):
                 got = qs[b, h, t]
-                assert got[5] == s_["nvalid"] and got[2] == s_["glob"] and got[4] == s_["rmax"]
+                # the device stores key positions of the rows' diagonals: gap + row without per-row positions
+                assert got[5] == s_["nvalid"] and got[2] == s_["glob"] and got[4] == (s_["rmax"] + (N - M) if s_["nvalid"] else -1)
                 if s_["nvalid"]:
-                    assert got[3] == s_["rmin"]
+                    assert got[3] == s_["rmin"] + (N - M)
                 if s_["lo"] <= s_["hi"]:
                     assert (got[0], got[1]) == (s_["lo"], s_["hi"])
                 else:
@@ -605,8 +655,40 @@ def test_varlen_causal_with_longer_key_sequences():
         ro, _, rdq, rdk, rdv = O.attention_autograd(sq(q), sk(k), sk(v), sq(do), True, None, None, None, 0)
         for name, got, ref, sl in (("o", out.detach(), ro, sq), ("dq", qd.grad, rdq, sq), ("dk", kd.grad, rdk, sk), ("dv", vd.grad, rdv, sk)):
             check_close(f"sequence {s} {name}", sl(got.float().cpu()), ref, quiet=True)
-    with pytest.raises(AssertionError):   # fewer keys than queries in a sequence
-        attention_varlen(qd, kd, vd, cuq.cuda(), torch.tensor([0, 10, 240, 245, 409, 486], dtype=torch.int32).cuda(), causal=True)
+
+
+def test_varlen_causal_sequence_with_fewer_keys_than_queries():
+    """A sequence with fewer keys than queries, bottom-right aligned: its first rows see no key
+    (O = 0, no gradient), the others the keys up to their diagonal; the whole packed problem against
+    the oracle with the same ids and positions, and the short sequence against its own closed form."""
+    from flash_mi355 import attention_varlen, varlen_ids, varlen_positions
+    from oracle import attention_oracle as O
+    lq, lk = [40, 30, 100], [40, 12, 164]
+    cuq = torch.tensor(np.concatenate([[0], np.cumsum(lq)]), dtype=torch.int32)
+    cuk = torch.tensor(np.concatenate([[0], np.cumsum(lk)]), dtype=torch.int32)
+    Tq, Tk, H, D = int(cuq[-1]), int(cuk[-1]), 2, 64
+    g = torch.Generator().manual_seed(29)
+    q, do = (torch.randn(Tq, H, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    k, v = (torch.randn(Tk, H, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    print("varlen causal, a sequence with fewer keys than queries", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cuq.cuda(), cuk.cuda(), causal=True)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    assert out[40:40 + 18].abs().max().item() == 0 and qd.grad[40:40 + 18].abs().max().item() == 0   # rows 0..17 of sequence 1: no key
+    t4 = lambda t: t.transpose(0, 1)[None]
+    eq = varlen_ids(cuq, Tq).view(1, 1, Tq).expand(1, H, Tq)
+    ek = varlen_ids(cuk, Tk).view(1, 1, Tk).expand(1, H, Tk)
+    ro, _, rdq, rdk, rdv = O.attention_autograd(t4(q), t4(k), t4(v), t4(do), True, None, eq, ek, 1,
+                                                qpos=varlen_positions(cuq, cuk, Tq).view(1, Tq))
+    for name, got, ref in (("o", out.detach(), ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        check_close(name, t4(got.float().cpu()), ref, quiet=True)
+    # rows 18..29 of sequence 1 against that sequence alone: local row 18 + t sees local keys 0..t
+    keep = torch.tril(torch.ones(12, 12, dtype=torch.bool))
+    qs, ks, vs = (t4(x).float() for x in (q[58:70], k[40:52], v[40:52]))
+    sc = (qs @ ks.transpose(-1, -2)) / math.sqrt(D)
+    ref = torch.softmax(sc.masked_fill(~keep, float("-inf")), -1) @ vs
+    assert (t4(out.detach()[58:70].float().cpu()) - ref).abs().max().item() <= TOL_O
 
 
 def test_varlen_cross_attention():

@@ -66,3 +66,24 @@ def test_varlen_ids_mark_sequences():
     for i in range(10):
         for j in range(10):
             assert bool(ids[i] == ids[j]) == (want[i] == want[j])
+
+
+def test_varlen_positions_align_sequences_bottom_right():
+    """Packed causal positions: row i of sequence s sits at packed key i + (end of the sequence's keys
+    - end of its queries), so the last query of every sequence sees exactly its last key; rows of a
+    sequence with fewer keys than queries that see nothing land before the sequence's first key."""
+    import torch
+    from flash_mi355 import varlen_positions
+    lq, lk = [4, 1, 0, 6, 3], [4, 9, 2, 8, 1]
+    cq = torch.tensor([0] + list(torch.tensor(lq).cumsum(0)), dtype=torch.int32)
+    ck = torch.tensor([0] + list(torch.tensor(lk).cumsum(0)), dtype=torch.int32)
+    pos = varlen_positions(cq, ck, int(cq[-1]))
+    assert pos.dtype == torch.int32 and pos.shape == (14,)
+    for s in range(5):
+        for t in range(lq[s]):
+            i = int(cq[s]) + t
+            want = int(ck[s]) + t + (lk[s] - lq[s])            # bottom-right: local row t sees local keys <= t + (lk - lq)
+            assert int(pos[i]) == max(want, -1)
+    assert int(pos[int(cq[4])]) < int(ck[4])                   # first rows of the last sequence (3 queries, 1 key): no key
+    same = varlen_positions(cq, cq, int(cq[-1]))
+    assert torch.equal(same, torch.arange(14, dtype=torch.int32))

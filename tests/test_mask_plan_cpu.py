@@ -57,3 +57,22 @@ def test_plan_is_sound(case, causal):
                 # the doc test passes everywhere; only causal / tail masking may remove elements
                 doc_only = O.keep_mask(M, N, False, eq[None, None], ek[None, None], 1)[0, 0]
                 assert doc_only[np.ix_(r, np.arange(kt * 64, min(N, (kt + 1) * 64)))].all()
+
+
+@settings(max_examples=40, deadline=None)
+@given(id_case(), st.integers(0, 2**31 - 1))
+def test_plan_is_sound_with_per_row_positions(case, seed):
+    """The same soundness property when every row carries its own causal position (arbitrary, not
+    even monotonic; -1 = the row sees nothing): summaries hold the smallest / largest position."""
+    M, N, eq, ek = case
+    rng = np.random.default_rng(seed)
+    pos = rng.integers(-1, N + 3, M)
+    perm, hdr, qs = P.plan_q(eq, M, pos)
+    ks = P.plan_k(ek, N)
+    keep = O.keep_mask(M, N, True, eq[None, None], ek[None, None], 1, qpos=pos[None])[0, 0]
+    for t, q in enumerate(qs):
+        r = perm[t * 64:(t + 1) * 64]
+        r = r[r >= 0]
+        for kt, k in enumerate(ks):
+            if len(r) and not P.visits(q, k, kt, True, 0):
+                assert not keep[np.ix_(r, np.arange(kt * 64, min(N, (kt + 1) * 64)))].any(), "a skipped tile pair holds a kept element"

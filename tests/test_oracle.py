@@ -323,6 +323,63 @@ def test_closed_form_with_window_matches_sdpa():
         assert (o - ref).abs().max().item() < 1e-5
 
 
+# ------------------------------------------------------------------ per-row causal positions
+def test_per_row_positions_brute_force_and_special_cases():
+    """keep_mask(qpos=...): element by element in Python loops (with ids and a window), the default
+    recovered by qpos = gap + i, and rows at -1 seeing nothing."""
+    rng = np.random.default_rng(5)
+    M, N = 9, 13
+    eq, ek = _ids(rng, 2, 2, M), _ids(rng, 2, 2, N)
+    pos = rng.integers(-1, N + 2, (2, M))
+    for window in (0, 1, 4):
+        got = np.broadcast_to(O.keep_mask(M, N, True, eq, ek, 1, window=window, qpos=pos), (2, 2, M, N))
+        for b in range(2):
+            for h in range(2):
+                for i in range(M):
+                    for j in range(N):
+                        c = pos[b, i] >= j and (not window or j > pos[b, i] - window)
+                        assert got[b, h, i, j] == bool(c and (eq[b, h, i] >= 0 or eq[b, h, i] == ek[b, h, j]))
+    base = (N - M) + np.arange(M)
+    assert np.array_equal(O.keep_mask(M, N, True, qpos=base[None]), O.keep_mask(M, N, True))
+    assert np.array_equal(O.keep_mask(M, N, True, window=3, qpos=base[None]), O.keep_mask(M, N, True, window=3))
+    assert not O.keep_mask(M, N, True, qpos=np.full((1, M), -1)).any()
+    assert O.keep_mask(M, N, True, qpos=np.full((1, M), N - 1)).all()
+    with pytest.raises(AssertionError):
+        O.keep_mask(M, N, False, qpos=base[None])
+    with pytest.raises(AssertionError):
+        O.keep_mask(M, N, True, prefix=2, qpos=base[None])
+
+
+def test_per_row_positions_align_every_packed_sequence_bottom_right():
+    """The case qpos exists for: a packed batch whose sequences have more keys than queries.  With the
+    negated sequence numbers as ids and qpos[i] = i + (end of the sequence's keys - end of its
+    queries), the packed mask is block diagonal and every block is the reference's rectangular causal
+    mask of that sequence alone (max(0, Lk - Lq) + i >= j, flash_triton.py:107,521); O, LSE and the
+    gradients of the packed problem equal those of the sequences taken one by one."""
+    lq, lk = [4, 1, 0, 6, 3], [4, 9, 2, 8, 5]
+    cq, ck = np.concatenate([[0], np.cumsum(lq)]), np.concatenate([[0], np.cumsum(lk)])
+    Tq, Tk = cq[-1], ck[-1]
+    eq = np.concatenate([np.full(n, -(s + 1)) for s, n in enumerate(lq)])[None, None]
+    ek = np.concatenate([np.full(n, -(s + 1)) for s, n in enumerate(lk)])[None, None]
+    qpos = np.concatenate([np.arange(cq[s], cq[s + 1]) + (ck[s + 1] - cq[s + 1]) for s in range(len(lq))])[None]
+    keep = O.keep_mask(Tq, Tk, True, eq, ek, 1, qpos=qpos)[0, 0]
+    want = np.zeros((Tq, Tk), bool)
+    for s in range(len(lq)):
+        want[cq[s]:cq[s + 1], ck[s]:ck[s + 1]] = O.keep_mask(lq[s], lk[s], True)[0, 0]
+    assert np.array_equal(keep, want)
+    q, k, v, do = _rand(1, 2, Tq, Tk, 8, seed=9)
+    o, lse, dq, dk, dv = O.attention_autograd(q, k, v, do, True, None, torch.from_numpy(eq).expand(1, 2, Tq),
+                                              torch.from_numpy(ek).expand(1, 2, Tk), 1, torch.float64, qpos=torch.from_numpy(qpos))
+    for s in range(len(lq)):
+        if lq[s] == 0:
+            assert dk[:, :, ck[s]:ck[s + 1]].abs().max() == 0 and dv[:, :, ck[s]:ck[s + 1]].abs().max() == 0
+            continue
+        sq, sk = slice(cq[s], cq[s + 1]), slice(ck[s], ck[s + 1])
+        ro, rl, rdq, rdk, rdv = O.attention_autograd(q[:, :, sq], k[:, :, sk], v[:, :, sk], do[:, :, sq], True, None, None, None, 0, torch.float64)
+        for got, ref in ((o[:, :, sq], ro), (lse[:, :, sq], rl), (dq[:, :, sq], rdq), (dk[:, :, sk], rdk), (dv[:, :, sk], rdv)):
+            assert (got - ref).abs().max().item() < 1e-12
+
+
 def test_storage_rounding_sets_the_gradient_error_floor():
     """What the reference's own rounding points (P, dS and the stored O in bf16; flash_triton.py:126,165,
     306,417,539) cost in the gradients, on the CPU.  With N(0,1) inputs at the default scale the exact

@@ -33,10 +33,10 @@ extern "C" const char* fa_error_string(int code) {
     case FA_ERR_NULLPTR: return "null pointer for a required operand";
     case FA_ERR_UNSUPPORTED_D: return "head dimension must be one of 16, 32, 64, 128";
     case FA_ERR_DTYPE: return "unsupported element or id type";
-    case FA_ERR_SHAPE: return "inconsistent sizes (H % Hk != 0, causal with N < M, or a size <= 0)";
+    case FA_ERR_SHAPE: return "inconsistent sizes (H % Hk != 0, causal with N < M and no qpos, or a size <= 0)";
     case FA_ERR_ALIGN: return "pointers must be 16-byte aligned and outer strides multiples of 16 bytes";
     case FA_ERR_STRIDE: return "innermost stride must be 1";
-    case FA_ERR_MODE: return "unknown score mode, doc mode without eq/ek, or window / prefix without causal (or both)";
+    case FA_ERR_MODE: return "unknown score mode, doc mode without eq/ek, window / prefix without causal (or both), or qpos without causal + ids (or with prefix)";
     case FA_ERR_WORKSPACE: return "workspace missing or too small";
     case FA_ERR_HIP: return "kernel launch failed";
     case FA_ERR_NOT_IMPLEMENTED: return "configuration not implemented";
@@ -50,7 +50,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if (p->dtype != FA_DTYPE_BF16 && p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_FP32) return FA_ERR_DTYPE;
   if (p->B <= 0 || p->H <= 0 || p->Hk <= 0 || p->M <= 0 || p->N <= 0) return FA_ERR_SHAPE;
   if (p->H % p->Hk != 0) return FA_ERR_SHAPE;
-  if (p->causal && p->N < p->M) return FA_ERR_SHAPE;
+  if (p->causal && p->N < p->M && p->qpos == nullptr) return FA_ERR_SHAPE;
   if (p->score_mode != FA_SCORE_MODE0_NOPE && p->score_mode != FA_SCORE_MODE1_DOC && p->score_mode != FA_SCORE_MODE2_BLOCK)
     return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE2_BLOCK) {
@@ -60,6 +60,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if ((p->flags & ~(FA_FLAG_DQ_DELTA | FA_FLAG_DEBUG_NO_PAIR_WAIT)) != 0) return FA_ERR_MODE;
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
   if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
+  if (p->qpos != nullptr && (!p->causal || p->score_mode != FA_SCORE_MODE1_DOC || p->prefix > 0 || p->qpos_stride < 0)) return FA_ERR_MODE;
   if (p->score_mode == FA_SCORE_MODE1_DOC) {
     if (p->eq == nullptr || p->ek == nullptr) return FA_ERR_MODE;
     if (p->id_dtype != FA_IDTYPE_I32 && p->id_dtype != FA_IDTYPE_I64) return FA_ERR_DTYPE;
@@ -68,6 +69,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->workspace_bytes < fa_workspace_bytes(p)) return FA_ERR_WORKSPACE;
   }
   if (stage == 2) return FA_OK;
+  if (p->qpos != nullptr && p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
   int rc;
   if ((rc = check_tensor(p->q, p->q_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
   if ((rc = check_tensor(p->k, p->k_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
@@ -114,6 +116,7 @@ static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratch
   a.pfx_m1 = p->prefix > 0 ? (p->prefix < p->N ? p->prefix : p->N) - 1 : -1;
   a.scale = p->sm_scale;
   a.scale_log2e = p->sm_scale * kLog2e;
+  a.ppos = nullptr; a.qpos = p->qpos; a.qp_bs = p->qpos_stride;
   a.eq32 = nullptr; a.ek32 = nullptr; a.perm = nullptr; a.peq = nullptr; a.qhdr = nullptr; a.qsum = nullptr; a.ksum = nullptr;
   a.sk_cnt = nullptr; a.sk_ml = nullptr; a.sk_o = nullptr;
   a.split_k = 1; a.split_tiles = 0;
@@ -136,6 +139,7 @@ static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratch
     a.ek32 = reinterpret_cast<const int*>(ws + w.off_ek32);
     a.perm = reinterpret_cast<const int*>(ws + w.off_perm);
     a.peq = reinterpret_cast<const int*>(ws + w.off_peq);
+    a.ppos = reinterpret_cast<const int*>(ws + w.off_ppos);
     a.qhdr = reinterpret_cast<const QHeader*>(ws + w.off_qhdr);
     a.qsum = reinterpret_cast<const IdSummary*>(ws + w.off_qsum);
     a.ksum = reinterpret_cast<const IdSummary*>(ws + w.off_ksum);

@@ -61,7 +61,7 @@ template <bool I64>
 __global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
                                                          int M, int Mp, int Pp, int nCh, int H1, int* __restrict__ eq32,
                                                          int* __restrict__ perm, int* __restrict__ peq,
-                                                         int* __restrict__ cnt) {
+                                                         int* __restrict__ ppos, int* __restrict__ cnt) {
   __shared__ int sh[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -82,6 +82,7 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict_
   for (int i = ch * kPlanChunk + tid; i < p_end; i += 256) {
     perm[bh * Pp + i] = -1;
     peq[bh * Pp + i] = 0;
+    ppos[bh * Pp + i] = -1;
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) c += __shfl_xor(c, off);
@@ -96,7 +97,8 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict_
 __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp, int nCh, int H1,
                                                            const int* __restrict__ eq32, const int* __restrict__ cnt,
                                                            int* __restrict__ perm, int* __restrict__ peq,
-                                                           QHeader* __restrict__ hdr) {
+                                                           int* __restrict__ ppos, const int* __restrict__ qpos, int64_t qp_bs,
+                                                           int gap, QHeader* __restrict__ hdr) {
   __shared__ int sh_l[4], sh_g[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -104,6 +106,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
   const int* eqp = eq32 + bh * Mp;
   int* pmp = perm + bh * Pp;
   int* pqp = peq + bh * Pp;
+  int* ppp = ppos + bh * Pp;
   int before = 0, nL = 0;
   for (int k = 0; k < nCh; ++k) {
     const int c = cnt[bh * nCh + k];
@@ -120,6 +123,8 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
     const int r = ch * kPlanChunk + k * 256 + tid;
     const bool valid = r < M;
     const int v = valid ? eqp[r] : 0;
+    // key position of the row's diagonal: the caller's, or the one offset of flash_triton.py:521
+    const int ps = !valid ? -1 : (qpos != nullptr ? clamp_pos(qpos[b * qp_bs + r]) : gap + r);
     const bool isL = valid && v < 0, isG = valid && v >= 0;
     const unsigned long long bl = __builtin_amdgcn_ballot_w64(isL), bg = __builtin_amdgcn_ballot_w64(isG);
     if (lane == 0) { sh_l[wave] = __builtin_popcountll(bl); sh_g[wave] = __builtin_popcountll(bg); }
@@ -131,8 +136,8 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
       if (w < wave) { offL += cl; offG += cg; }
       totL += cl; totG += cg;
     }
-    if (isL) { const int pos = baseL + offL + __builtin_popcountll(bl & lt); pmp[pos] = r; pqp[pos] = v; }
-    if (isG) { const int pos = baseG + offG + __builtin_popcountll(bg & lt); pmp[pos] = r; pqp[pos] = v; }
+    if (isL) { const int pos = baseL + offL + __builtin_popcountll(bl & lt); pmp[pos] = r; pqp[pos] = v; ppp[pos] = ps; }
+    if (isG) { const int pos = baseG + offG + __builtin_popcountll(bg & lt); pmp[pos] = r; pqp[pos] = v; ppp[pos] = ps; }
     baseL += totL; baseG += totG;
     __syncthreads();
   }
@@ -146,8 +151,9 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
 // Step 3: one wave per 64 entries of the permuted order: id / row-index summary, and the range
 // [kfirst, klast] of key tiles the entry's rows can need (by the key summaries and the causal
 // bound), so that the compute kernels start their tile search in the right place.
-__global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal_gap, int kend_min,
+__global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs, int H1, int HK1, int causal, int kend_min,
                                                         const int* __restrict__ perm, const int* __restrict__ peq,
+                                                        const int* __restrict__ ppos,
                                                         const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum,
                                                         int* __restrict__ sk_cnt, int n_sk) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -160,20 +166,21 @@ __global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs
   const int64_t bh = int64_t(b) * H1 + h;
   const int row = perm[bh * Pp + t * kSumRows + lane];
   const int v = peq[bh * Pp + t * kSumRows + lane];
+  const int ps = ppos[bh * Pp + t * kSumRows + lane];
   const bool valid = row >= 0;
   const bool local = valid && v < 0;
   IdSummary s;
   s.lo = wave_min(local ? v : 0x7fffffff);
   s.hi = wave_max(local ? v : (int)0x80000000);
-  s.rmin = wave_min(valid ? row : 0x7fffffff);
-  s.rmax = wave_max(valid ? row : -1);
+  s.rmin = wave_min(valid ? ps : 0x7fffffff);
+  s.rmax = wave_max(valid ? ps : -1);
   s.glob = __builtin_amdgcn_ballot_w64(valid && v >= 0) != 0 ? 1 : 0;
   s.nvalid = __builtin_popcountll(__builtin_amdgcn_ballot_w64(valid));
   int kfirst = 0x7fffffff, klast = -1;
   if (H1 == HK1) {  // ids of both sides stored per the same heads: narrow the key range
     const IdSummary* ks = ksum + bh * nKs;
     // kend_min: key tiles of a prefix that every row sees whatever its causal bound
-    const int kend = causal_gap >= 0 ? min(nKs, max((causal_gap + s.rmax) / kSumRows + 1, kend_min)) : nKs;
+    const int kend = causal ? min(nKs, max(s.rmax / kSumRows + 1, kend_min)) : nKs;
     for (int k0 = 0; k0 < kend; k0 += 64) {
       const int k = k0 + lane;
       bool cand = false;
@@ -201,6 +208,7 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
   int* ek32 = reinterpret_cast<int*>(ws + w.off_ek32);
   int* perm = reinterpret_cast<int*>(ws + w.off_perm);
   int* peq = reinterpret_cast<int*>(ws + w.off_peq);
+  int* ppos = reinterpret_cast<int*>(ws + w.off_ppos);
   int* cnt = reinterpret_cast<int*>(ws + w.off_cnt);
   QHeader* hdr = reinterpret_cast<QHeader*>(ws + w.off_qhdr);
   IdSummary* qsum = reinterpret_cast<IdSummary*>(ws + w.off_qsum);
@@ -219,15 +227,16 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
     const int64_t* st = p->eq_stride;
     dim3 grid(w.nCh, w.Hq1, p->B);
     if (i64)
-      hipLaunchKernelGGL(plan_count_kernel<true>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, cnt);
+      hipLaunchKernelGGL(plan_count_kernel<true>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, ppos, cnt);
     else
-      hipLaunchKernelGGL(plan_count_kernel<false>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, cnt);
-    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(plan_scatter_kernel, grid, dim3(256), 0, s, p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, cnt, perm, peq, hdr);
+      hipLaunchKernelGGL(plan_count_kernel<false>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, ppos, cnt);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     const int gap = p->N > p->M ? p->N - p->M : 0;
+    hipLaunchKernelGGL(plan_scatter_kernel, grid, dim3(256), 0, s, p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, cnt, perm, peq, ppos,
+                       p->causal ? p->qpos : nullptr, p->qpos_stride, gap, hdr);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
-                       p->causal ? gap : -1, p->prefix > 0 ? ((p->prefix < p->N ? p->prefix : p->N) - 1) / kSumRows + 1 : 0, perm, peq, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
+                       p->causal ? 1 : 0, p->prefix > 0 ? ((p->prefix < p->N ? p->prefix : p->N) - 1) / kSumRows + 1 : 0, perm, peq, ppos, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
                        p->B * p->H * w.split.tiles);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
@@ -244,7 +253,8 @@ __global__ __launch_bounds__(256) void mask_dump_kernel(const KArgs a, uint8_t* 
     const int ek_j = DOC ? a.ek32[b * a.ek_bs + h * a.ek_hs + j] : 0;
     for (int i = blockIdx.y; i < a.M; i += gridDim.y) {
       const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + i] : 0;
-      bool keep = keep_elem<CAUSAL, DOC>(i, j, a.gap, a.N, eq_i, ek_j, a.win, a.pfx_m1);
+      const int pos_i = (DOC && CAUSAL && a.qpos != nullptr) ? clamp_pos(a.qpos[b * a.qp_bs + i]) : a.gap + i;
+      bool keep = keep_elem<CAUSAL, DOC>(pos_i, j, a.N, eq_i, ek_j, a.win, a.pfx_m1);
       if (!DOC && a.bmask != nullptr)
         keep = keep && a.bmask[b * a.bm_bs + h * a.bm_hs + int64_t(i / FA_MASK_BLOCK) * a.bm_rs + j / FA_MASK_BLOCK] != 0;
       out[(int64_t(bh) * a.M + i) * a.N + j] = keep ? 1 : 0;

@@ -101,8 +101,13 @@ void bwd_dkdv_kernel(const KArgs a) {
   const float c = a.scale_log2e;
   // rows that may see this lane's key: [row_lo, row_lo + row_span)
   // (causal: from the diagonal on, or from row 0 for a key of the prefix; sliding window: `win` rows)
-  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - a.gap)) : 0;
-  const int row_hi = CAUSAL ? min(a.M - 1, key - a.gap + a.win - 1) : a.M - 1;
+  // Without ids a row is named by its index r and its diagonal sits at key gap + r; with ids rows are
+  // named by the diagonal position the mask plan stored for them (gap + row, or the caller's per-row
+  // position), so the offset is 0 and the names run up to kPosMax.
+  const int gk = DOC ? 0 : a.gap;
+  const int rcap = DOC ? kPosMax : a.M - 1;
+  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - gk)) : 0;
+  const int row_hi = CAUSAL ? min(rcap, key - gk + a.win - 1) : rcap;
   const unsigned row_span = (key < a.N && row_hi >= row_lo) ? (unsigned)(row_hi - row_lo + 1) : 0u;
 
   // per query head state (set at the top of the head loop)
@@ -112,6 +117,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   int wk_lo = 0, wk_hi = 0;   // id interval of this wave's 32 keys
   const int* eqp = nullptr;
   const int* pmp = nullptr;
+  const int* ppp = nullptr;   // diagonal positions in the permuted order
   const IdSummary* qsum = nullptr;
 
   Loader ldQ, ldO;
@@ -171,7 +177,7 @@ void bwd_dkdv_kernel(const KArgs a) {
       if (wave == 0) glb_load_lds4(lsep + r, aux);
       if (wave == 1) glb_load_lds4(delp + r, aux + 256);
       if (wave == 2) glb_load_lds4(eqp + r, aux + 512);
-      if (wave == 3) glb_load_lds4(pmp + tile * BQ + lane, aux + 768);
+      if (wave == 3) glb_load_lds4(ppp + tile * BQ + lane, aux + 768);
     }
   };
 
@@ -185,7 +191,7 @@ void bwd_dkdv_kernel(const KArgs a) {
                     __attribute__((always_inline)) {
     const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0, has_glob = (flags & TF_GLOB) != 0;
     if (need_lim) {
-      // row index inside [first row that may see this key, M); padding rows are -1.  The four index
+      // row name (index, or diagonal position with ids) inside [first that may see this key, last]; padding rows are -1.  The four index
       // vectors are requested together: one LDS round trip instead of four serial ones.
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
       i32x4 rowv[4];
@@ -458,14 +464,15 @@ void bwd_dkdv_kernel(const KArgs a) {
     ldO.init(reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs, a.do_rs, a.M);
     int gk_lo = 0, gk_hi = 0;   // id interval of the workgroup's 128 keys
     int nQtiles = (a.M + BQ - 1) / BQ;
-    int first = CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - a.gap) / BQ) : 0;
+    int first = CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - gk) / BQ) : 0;
     // sliding window: the last row that sees a key of this workgroup
-    const int wg_rhi = CAUSAL ? min(a.M - 1, n0 + BK - 1 - a.gap + a.win - 1) : a.M - 1;
-    if (CAUSAL) nQtiles = min(nQtiles, max(0, wg_rhi + 1 + BQ - 1) / BQ);
+    const int wg_rhi = CAUSAL ? min(rcap, n0 + BK - 1 - gk + a.win - 1) : rcap;
+    if (CAUSAL && !DOC) nQtiles = min(nQtiles, max(0, wg_rhi + 1 + BQ - 1) / BQ);
     if (DOC) {
       ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
       eqp = a.eq32 + b * a.eq_bs + h * a.eq_hs;
       pmp = a.perm + b * a.pm_bs + h * a.pm_hs;
+      ppp = a.ppos + b * a.pm_bs + h * a.pm_hs;
       qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
       const IdSummary* ks = a.ksum + b * a.ks_bs + h * a.ks_hs;
       const IdSummary s0 = ks[n0 / kSumRows];
@@ -507,10 +514,10 @@ void bwd_dkdv_kernel(const KArgs a) {
           none = (b0 | b1) == 0;
         }
       } else {
-        skip = (nw >= a.N) || (CAUSAL && ((a.gap + qs.rmax < nw && nw > a.pfx_m1) || a.gap + qs.rmin - a.win + 1 > nw + 31)) ||
+        skip = (nw >= a.N) || (CAUSAL && ((qs.rmax < nw && nw > a.pfx_m1) || qs.rmin - a.win + 1 > nw + 31)) ||
                !doc_may_keep(qs.lo, qs.hi, qs.glob, wk_lo, wk_hi);
         lim = (qs.nvalid < BQ) || (nw + 32 > a.N) ||
-              (CAUSAL && ((a.gap + qs.rmin < nw + 31 && nw + 31 > a.pfx_m1) || a.gap + qs.rmax - a.win + 1 > nw));
+              (CAUSAL && ((qs.rmin < nw + 31 && nw + 31 > a.pfx_m1) || qs.rmax - a.win + 1 > nw));
         doc = !doc_all_keep(qs.lo, qs.hi, wk_lo, wk_hi);
         glob = qs.glob != 0;
         // one local id for the whole tile (padding rows aside, which the row-range mask drops):
@@ -522,7 +529,7 @@ void bwd_dkdv_kernel(const KArgs a) {
                         (none ? TF_NONE : 0), qs.lo);
     };
     TileIter it;
-    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL && n0 > a.pfx_m1 ? n0 - a.gap : (int)0x80000000,
+    it.init_queries(first, nQtiles, qsum, gk_lo, gk_hi, CAUSAL && n0 > a.pfx_m1 ? n0 - gk : (int)0x80000000,
                     CAUSAL ? wg_rhi : 0x7fffffff, dec);
     if (gi > 0) __syncthreads();  // the previous head's last tile may still be read from LDS
 

@@ -91,6 +91,11 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget 
 
 constexpr int kPairSpinDefault = 1 << 14;
 
+// Key position of a row's diagonal as the kernels use it: at least -1 (the row sees nothing), and
+// small enough that position + window never overflows.
+constexpr int kPosMax = 0x3fffffff;
+FA_HD int clamp_pos(int v) { return v < -1 ? -1 : (v > kPosMax ? kPosMax : v); }
+
 struct bf16_t {};
 struct fp16_t {};
 
@@ -181,10 +186,11 @@ FA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 // ---------------------------------------------------------------------------
 //   window : j > gap + i - win (win = 0x3fffffff: off)    sliding window, causal only
 //   prefix : the causal term also holds for j <= pfx_m1   prefix-LM (pfx_m1 = -1: off)
+//   pos_i  : key position of row i's diagonal: gap + i, or the caller's per-row position (fa_params.qpos)
 template <bool CAUSAL, bool DOC>
-FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j, int win, int pfx_m1) {
+FA_DEV bool keep_elem(int pos_i, int j, int N, int eq_i, int ek_j, int win, int pfx_m1) {
   bool keep = j < N;
-  if (CAUSAL) keep = keep && ((gap + i >= j) || (j <= pfx_m1)) && (j > gap + i - win);
+  if (CAUSAL) keep = keep && ((pos_i >= j) || (j <= pfx_m1)) && (j > pos_i - win);
   if (DOC) keep = keep && ((eq_i >= 0) || (eq_i == ek_j));
   return keep;
 }
@@ -203,7 +209,8 @@ FA_DEV bool keep_elem(int i, int j, int gap, int N, int eq_i, int ek_j, int win,
 struct IdSummary {
   int lo, hi;      // min / max id: query side over local rows (lo > hi if none), key side over all keys
   int glob;        // query side: 1 if the tile holds global rows
-  int rmin, rmax;  // query side: smallest / largest original row index of the tile (rmax = -1 if empty)
+  int rmin, rmax;  // query side: smallest / largest diagonal position (ppos) of the tile's rows (rmax = -1 if empty);
+                   // key side: first / last key of the tile
   int nvalid;      // query side: rows of the tile that exist
   int kfirst, klast;  // query side: first / last key tile (of 64 keys) the rows can need (klast < kfirst: none)
 };
@@ -239,6 +246,9 @@ struct KArgs {
   const int* ek32;        // [B, Hk', Np]
   const int* perm;        // [B, Hq', Pp]   permuted order -> original row (or -1)
   const int* peq;         // [B, Hq', Pp]   id of that row
+  const int* ppos;        // [B, Hq', Pp]   key position of that row's diagonal (gap + row, or the caller's qpos), -1 for padding
+  const int* qpos;        // the caller's per-row positions [B, M] in natural order, or null (mask dump)
+  int64_t qp_bs;
   const QHeader* qhdr;    // [B, Hq']
   const IdSummary* qsum;  // [B, Hq', nQs]  per 64 entries of the permuted order
   const IdSummary* ksum;  // [B, Hk', nKs]  per 64 keys
@@ -284,7 +294,7 @@ struct WsLayout {
   int Pp;                 // length of the permuted order
   int nQs, nKs;
   int nCh;                // row chunks of the partition kernels
-  uint64_t off_eq32, off_ek32, off_perm, off_peq, off_cnt, off_qhdr, off_qsum, off_ksum;  // bytes
+  uint64_t off_eq32, off_ek32, off_perm, off_peq, off_ppos, off_cnt, off_qhdr, off_qsum, off_ksum;  // bytes
   uint64_t off_sk_cnt, off_sk_ml, off_sk_o, total;
   uint64_t plan_bytes;   // leading part that carries state from the plan to the kernels; the rest is scratch
   SplitCfg split;        // split of long key ranges this layout has scratch for
@@ -306,6 +316,7 @@ inline WsLayout ws_layout(const fa_params* p, uint64_t split_budget = kSplitScra
   w.off_ek32 = take(uint64_t(p->B) * w.Hk1 * w.Np * 4);
   w.off_perm = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
   w.off_peq = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
+  w.off_ppos = take(uint64_t(p->B) * w.Hq1 * w.Pp * 4);
   w.nCh = (w.Mp + 1023) / 1024;
   w.off_cnt = take(uint64_t(p->B) * w.Hq1 * w.nCh * 4);
   w.off_qhdr = take(uint64_t(p->B) * w.Hq1 * sizeof(QHeader));

@@ -261,7 +261,11 @@ struct QTileCtx {
   int row;    // original row index of this lane's query (lanes l and l^32 share it), -1 if none
   int rowc;   // row clamped into [0, M) for loads
   int eq_i;
-  int w_lo, w_hi, w_glob, w_rmin, w_rmax;  // this wave's 32 rows
+  // Causal terms are written in key positions: the diagonal of row i sits at key gp + r, where without ids
+  // r is the row index and gp = gap, and with ids r is the position the mask plan stored for the row
+  // (gap + row, or the caller's per-row position) and gp = 0.
+  int gp;
+  int w_lo, w_hi, w_glob, w_rmin, w_rmax;  // this wave's 32 rows (rmin / rmax: smallest / largest r)
   int g_lo, g_hi, g_glob, g_rmin, g_rmax;  // the workgroup's 128 rows
   int g_kfirst, g_klast;                   // key tiles (of 64) those rows can need, from the mask plan
   int lim_i;                               // last key this lane's row may see (causal / prefix and length limit)
@@ -281,12 +285,15 @@ struct QTileCtx {
     eq_i = 0; ekp = nullptr; ksum = nullptr;
     w_lo = 0; w_hi = -1; w_glob = 1; g_lo = 0; g_hi = -1; g_glob = 1;
     g_kfirst = 0; g_klast = 0x3fffffff;
+    gp = DOC ? 0 : a.gap;
+    int posc;   // r of this lane's row, 0 if none
     if (!DOC) {
       const int m0 = tile * 128, mw = m0 + wave * 32;
       row = mw + lq < a.M ? mw + lq : -1;
       w_rmin = mw; w_rmax = min(mw + 31, a.M - 1);
       if (w_rmax < w_rmin) w_rmax = -1;
       g_rmin = m0; g_rmax = min(m0 + 127, a.M - 1);
+      posc = row >= 0 ? row : 0;
     } else {
       ekp = a.ek32 + b * a.ek_bs + h * a.ek_hs;
       ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
@@ -295,6 +302,7 @@ struct QTileCtx {
       const int64_t pos = b * a.pm_bs + h * a.pm_hs + tile * 128 + wave * 32 + lq;
       row = a.perm[pos];     // issued together with the summaries: no dependent load chain
       eq_i = a.peq[pos];
+      const int ps = a.ppos[pos];
       if (s0.nvalid + s1.nvalid == 0) {  // no rows: every decision below says "skip"
         row = -1; rowc = 0; eq_i = 0; w_rmin = 0x7fffffff; w_rmax = -1; w_glob = 0;
         g_lo = 0x7fffffff; g_hi = (int)0x80000000; g_glob = 0; g_rmin = 0x7fffffff; g_rmax = -1;
@@ -305,7 +313,8 @@ struct QTileCtx {
       g_kfirst = min(s0.kfirst, s1.kfirst); g_klast = max(s0.klast, s1.klast);
       const bool local = (eq_i < 0) && (row >= 0);
       int lo = local ? eq_i : 0x7fffffff, hi = local ? eq_i : (int)0x80000000;
-      int rmin = row >= 0 ? row : 0x7fffffff, rmax = row;
+      int rmin = row >= 0 ? ps : 0x7fffffff, rmax = row >= 0 ? ps : -1;
+      posc = row >= 0 ? ps : 0;
 #pragma unroll
       for (int off = 16; off >= 1; off >>= 1) {
         lo = min(lo, __shfl_xor(lo, off));
@@ -317,21 +326,21 @@ struct QTileCtx {
       w_glob = __builtin_amdgcn_ballot_w64(eq_i >= 0 && row >= 0) != 0;
     }
     rowc = row >= 0 ? row : 0;
-    lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;
-    w_limmin = CAUSAL ? min(max(a.gap + w_rmin, a.pfx_m1), a.N - 1) : a.N - 1;
-    low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;
-    w_lowmin = CAUSAL && w_rmax >= 0 ? a.gap + w_rmin - a.win + 1 : -0x3fffffff;
-    w_lowmax = CAUSAL && w_rmax >= 0 ? a.gap + w_rmax - a.win + 1 : -0x3fffffff;
+    lim_i = CAUSAL ? min(max(gp + posc, a.pfx_m1), a.N - 1) : a.N - 1;
+    w_limmin = CAUSAL ? min(max(gp + w_rmin, a.pfx_m1), a.N - 1) : a.N - 1;
+    low_i = CAUSAL ? gp + posc - a.win + 1 : -0x3fffffff;
+    w_lowmin = CAUSAL && w_rmax >= 0 ? gp + w_rmin - a.win + 1 : -0x3fffffff;
+    w_lowmax = CAUSAL && w_rmax >= 0 ? gp + w_rmax - a.win + 1 : -0x3fffffff;
     glob_i = eq_i >= 0;
     return true;
   }
   // range [first, last) of 64-key tiles the workgroup has to look at
   FA_DEV int first_tile(const KArgs& a) const {
     const int f = g_kfirst < 0x3fffffff ? g_kfirst : 0;
-    return CAUSAL && g_rmax >= 0 ? max(f, max(0, a.gap + g_rmin - a.win + 1) / 64) : f;   // sliding window
+    return CAUSAL && g_rmax >= 0 ? max(f, max(0, gp + g_rmin - a.win + 1) / 64) : f;   // sliding window
   }
   FA_DEV int last_tile(const KArgs& a) const {
-    const int hi_key = CAUSAL ? min(a.N, max(a.gap + g_rmax, a.pfx_m1) + 1) : a.N;
+    const int hi_key = CAUSAL ? min(a.N, max(gp + g_rmax, a.pfx_m1) + 1) : a.N;
     return min((hi_key + 63) / 64, g_klast + 1);
   }
 
@@ -340,7 +349,7 @@ struct QTileCtx {
   //   TF_LIM  : some pair fails the causal / length limit  -> mask_lim
   //   TF_DOC  : some pair may fail the id test             -> mask_doc
   FA_DEV int decide(const KArgs& a, int n0, int BN, int k_lo, int k_hi) const {
-    bool skip = (w_rmax < 0) || (CAUSAL && (n0 > max(a.gap + w_rmax, a.pfx_m1) || n0 + BN - 1 < w_lowmin));
+    bool skip = (w_rmax < 0) || (CAUSAL && (n0 > max(gp + w_rmax, a.pfx_m1) || n0 + BN - 1 < w_lowmin));
     const bool need_lim = n0 + BN - 1 > w_limmin || n0 < w_lowmax;
     bool need_doc = false;
     if (DOC) {

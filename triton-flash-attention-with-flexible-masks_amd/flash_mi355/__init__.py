@@ -6,7 +6,7 @@
 The four public names match the reference module ``flash_triton``.
 """
 from .api import (SCORE_FUNC_MODE0_NOPE, SCORE_FUNC_MODE1_DOC, SCORE_FUNC_MODE2_BLOCK, FlashAttention, FlashAttentionWithLse, attention,
-                  attention_varlen, attention_with_lse, mask_dump, maybe_contiguous, varlen_ids)
+                  attention_varlen, attention_with_lse, mask_dump, maybe_contiguous, varlen_ids, varlen_positions)
 
 __all__ = ["attention", "FlashAttention", "FlashAttentionWithLse", "SCORE_FUNC_MODE0_NOPE", "SCORE_FUNC_MODE1_DOC",
-           "attention_with_lse", "attention_varlen", "varlen_ids", "mask_dump", "maybe_contiguous"]
+           "attention_with_lse", "attention_varlen", "varlen_ids", "varlen_positions", "mask_dump", "maybe_contiguous"]

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libflash_mi355.so"
 
-FA_ABI_VERSION = 5
+FA_ABI_VERSION = 6
 FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
 FA_SCORE_MODE2_BLOCK = 2
@@ -46,6 +46,7 @@ class FaParams(Structure):
         ("B", c_int32), ("H", c_int32), ("Hk", c_int32), ("M", c_int32), ("N", c_int32), ("D", c_int32),
         ("causal", c_int32), ("score_mode", c_int32), ("dtype", c_int32), ("id_dtype", c_int32),
         ("sm_scale", c_float), ("flags", c_int32), ("window", c_int32), ("prefix", c_int32),
+        ("qpos", c_void_p), ("qpos_stride", c_int64),
     ]
 
 

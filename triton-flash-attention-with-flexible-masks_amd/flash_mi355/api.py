@@ -51,7 +51,7 @@ def _stream_ptr(device) -> int:
 class _Plan:
     """fa_params filled in for one problem, plus the tensors that keep its pointers alive."""
 
-    def __init__(self, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
+    def __init__(self, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0, qpos=None):
         B, H, M, D = q.shape
         N, Hk = k.shape[2], k.shape[1]
         p = _cabi.FaParams()
@@ -74,6 +74,10 @@ class _Plan:
             _set3(p.eq_stride, eq); _set3(p.ek_stride, ek)
             p.id_dtype = _ID_DTYPES[eq.dtype]
             self.keep += [eq, ek]
+        if qpos is not None:   # int32 [B | 1, M], row stride 1
+            p.qpos = qpos.data_ptr()
+            p.qpos_stride = qpos.stride(0) if qpos.shape[0] > 1 else 0
+            self.keep += [qpos]
         self.p = p
         self.workspace = None
 
@@ -127,7 +131,7 @@ class _Impl:
     """Forward and backward shared by the two autograd functions below."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0, qpos=None):
         # -- checks of flash_triton.py:510-530, same order and messages --
         Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
         assert Dq == Dk and Dk == Dv, "feature size of q, k, v should be equal"
@@ -138,7 +142,7 @@ class _Impl:
         assert Hk == Hv, "num of heads in k and v should be equal"
         assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
         num_groups = H // Hk
-        assert (N >= M) or (not causal), "KV length should be larger than M length in causal mode!"
+        assert (N >= M) or (not causal) or (qpos is not None), "KV length should be larger than M length in causal mode!"
         MN_GAP = max(0, N - M)
         if sm_scale is None:
             sm_scale = 1. / math.sqrt(D)
@@ -180,11 +184,18 @@ class _Impl:
                 zero = torch.zeros((1, 1, 1), dtype=torch.int32, device=q.device)   # every stride 0: one id for all
                 eq, ek = zero.expand(B, H, M), zero.expand(B, H, N)
                 score_func_mode = SCORE_FUNC_MODE1_DOC
+        if qpos is not None:
+            assert causal and score_func_mode == SCORE_FUNC_MODE1_DOC and not prefix, \
+                "qpos (per-row causal positions) needs causal=True and eq / ek, and excludes prefix"
+            assert qpos.dim() == 2 and qpos.shape[0] in (1, B) and qpos.shape[1] == M and not qpos.dtype.is_floating_point, \
+                "qpos must be an integer tensor [bs|1, Lq]"
+            _check_same_device(q, qpos=qpos)
+            qpos = qpos.to(torch.int32).contiguous()
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
 
         L = _cabi.lib()
         with torch.cuda.device(q.device):
-            plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
+            plan = _Plan(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
             Out = torch.empty_like(q)   # q's layout when q is dense (flash_triton.py:539), contiguous otherwise
             lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
             p = plan.p
@@ -192,7 +203,7 @@ class _Impl:
             _set4(p.o_stride, Out)
             plan.ensure_workspace(q.device)
             _cabi.check(L.fa_fwd(ctypes.byref(p), _stream_ptr(q.device)), "fa_fwd")
-        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.plan_state())
+        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.plan_state(), qpos)
         ctx.sm_scale = sm_scale
         ctx.causal = causal
         ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
@@ -201,7 +212,7 @@ class _Impl:
 
     @staticmethod
     def backward(ctx, do, dlse):
-        q, k, v, o, lse, eq, ek, workspace = ctx.saved_tensors
+        q, k, v, o, lse, eq, ek, workspace, qpos = ctx.saved_tensors
         B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
         score_func_mode, window, prefix = ctx.score_func_info
         L = _cabi.lib()
@@ -210,7 +221,7 @@ class _Impl:
         do = _aligned(maybe_contiguous(do))
         _check_same_device(q, do=do, dlse=dlse)
         with torch.cuda.device(q.device):
-            plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix)
+            plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
             p = plan.p
             if workspace is not None:   # the forward's mask plan is reused as is
                 plan.restore(workspace, q.device)
@@ -238,7 +249,7 @@ class _Impl:
                     delta.sub_(torch.where(torch.isinf(lse), torch.zeros_like(lse), dlse.to(torch.float32)))
                 _cabi.check(L.fa_bwd_dkdv(ctypes.byref(p), stream), "fa_bwd_dkdv")
                 _cabi.check(L.fa_bwd_dq(ctypes.byref(p), stream), "fa_bwd_dq")
-        return dq, dk, dv, None, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
 _forward, _backward = _Impl.forward, _Impl.backward
@@ -248,8 +259,8 @@ class FlashAttention(torch.autograd.Function):
     """Mirror of the reference autograd function (flash_triton.py:506-638)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
-        return _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)[0]
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0, qpos=None):
+        return _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix, qpos)[0]
 
     @staticmethod
     def backward(ctx, do):
@@ -262,8 +273,8 @@ class FlashAttentionWithLse(torch.autograd.Function):
     entry point returns Out only, flash_triton.py:564)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0):
-        out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
+    def forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window=0, prefix=0, qpos=None):
+        out, lse = _forward(ctx, q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
         ctx.set_materialize_grads(False)   # a result that is not used arrives as None, not as zeros
         return out, lse * math.log(2.0)
 
@@ -280,26 +291,29 @@ def _block_args(block_mask, eq, ek, score_func_mode):
 
 
 def attention(q, k, v, causal=False, sm_scale=None, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE,
-              *, window=0, prefix=0, block_mask=None):
+              *, window=0, prefix=0, block_mask=None, qpos=None):
     """flash_triton.py:640-641.  Keyword-only additions (no counterpart in the reference):
     window = W: sliding window, a row sees only its last W keys up to the diagonal (causal only);
     prefix = P: prefix-LM, the first P keys are seen by every row (causal only, excludes window);
     block_mask: block-sparse attention -- a bool / integer tensor [bs|1, H|1, ceil(Lq/64), ceil(Lk/64)];
     a (row, key) pair is kept iff its 64 x 64 block is non-zero (and the causal terms hold); blocks that
-    are switched off are never visited.  Excludes eq / ek."""
+    are switched off are never visited.  Excludes eq / ek.
+    qpos: per-row causal positions, an integer tensor [bs|1, Lq] -- row i has its diagonal at key
+    qpos[i] (it sees keys j <= qpos[i]) instead of max(0, Lk - Lq) + i; needs causal=True and eq / ek
+    (the ids confine a row to its sequence, qpos aligns each sequence on its own), excludes prefix."""
     eq, ek, score_func_mode = _block_args(block_mask, eq, ek, score_func_mode)
-    return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
+    return FlashAttention.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
 
 
 # ---------------------------------------------------------------------------
 # Accessors for tests and benchmarks (not part of the reference's surface).
 # ---------------------------------------------------------------------------
 def attention_with_lse(q, k, v, causal=False, sm_scale=None, eq=None, ek=None,
-                       score_func_mode=SCORE_FUNC_MODE0_NOPE, *, window=0, prefix=0, block_mask=None):
+                       score_func_mode=SCORE_FUNC_MODE0_NOPE, *, window=0, prefix=0, block_mask=None, qpos=None):
     """(O, LSE) with LSE in natural-log units (-inf for rows without a kept key); differentiable
     through both results."""
     eq, ek, score_func_mode = _block_args(block_mask, eq, ek, score_func_mode)
-    return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix)
+    return FlashAttentionWithLse.apply(q, k, v, causal, sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
 
 
 def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
@@ -311,23 +325,17 @@ def varlen_ids(cu_seqlens: torch.Tensor, total: int) -> torch.Tensor:
     return (-(seq + 1)).to(torch.int32)
 
 
-def _varlen_causal_by_sequence(q, k, v, cu_seqlens_q, cu_seqlens_k, sm_scale, window):
-    """Causal packed batch whose query and key boundaries differ: one operator call per sequence on
-    [1, H, len, D] views of the packed tensors (bottom-right aligned, so a sequence needs at least
-    as many keys as queries, flash_triton.py:520)."""
-    assert cu_seqlens_q.shape == cu_seqlens_k.shape, "cu_seqlens_q and cu_seqlens_k must describe the same sequences"
-    cq, ck = cu_seqlens_q.tolist(), cu_seqlens_k.tolist()
-    assert cq[0] == 0 and ck[0] == 0 and cq[-1] == q.shape[0] and ck[-1] == k.shape[0], "cu_seqlens must span the packed tensors"
-    outs = []
-    for s in range(len(cq) - 1):
-        qs = q[cq[s]:cq[s + 1]]
-        if qs.shape[0] == 0:
-            continue
-        ks, vs = k[ck[s]:ck[s + 1]], v[ck[s]:ck[s + 1]]
-        assert ks.shape[0] >= qs.shape[0], f"sequence {s}: causal attention needs at least as many keys as queries"
-        q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (qs, ks, vs))
-        outs.append(attention(q4, k4, v4, True, sm_scale, window=window).squeeze(0).transpose(0, 1))
-    return torch.cat(outs, 0) if outs else torch.empty_like(q)
+def varlen_positions(cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, total_q: int) -> torch.Tensor:
+    """Causal positions of a packed batch whose query and key boundaries differ: every sequence is
+    aligned bottom-right on its own (its last query sees its last key, flash_triton.py:521 applied per
+    sequence), so packed row i of sequence s has its diagonal at packed key i + (cu_k[s+1] - cu_q[s+1]).
+    A sequence with fewer keys than queries leaves its first rows without a key (positions before the
+    sequence's first key; output 0).  int32, shape [total_q]; computed on the device, no host sync."""
+    pos = torch.arange(total_q, device=cu_seqlens_q.device, dtype=torch.int64)
+    nseq = cu_seqlens_q.numel() - 1
+    seq = torch.bucketize(pos, cu_seqlens_q[1:].contiguous().to(torch.int64), right=True).clamp_(max=max(nseq - 1, 0))
+    shift = (cu_seqlens_k[1:].to(torch.int64) - cu_seqlens_q[1:].to(torch.int64))[seq]
+    return (pos + shift).clamp_(min=-1).to(torch.int32)
 
 
 def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_scale=None, *, window=0):
@@ -338,30 +346,31 @@ def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_
 
     The packed batch IS the document mask of the operator: one (batch) row of total_* tokens whose
     ids are the negated sequence numbers, so no padding and no copy -- q, k, v are passed as
-    [1, H, total, D] views.  That holds for every non-causal case and for causal self-attention
-    (cu_seqlens_k equal to cu_seqlens_q: the causal bound of the packed row and of every sequence
-    coincide).  Causal with different boundaries (queries that are the tail of a longer key
-    sequence: chunked prefill, decoding) aligns every sequence bottom-right on its own, which is
-    not one offset of the packed row: those sequences are launched one by one, each as the
-    rectangular causal case of the operator (flash_triton.py:520-521), still without a copy.
+    [1, H, total, D] views, one launch per kernel whatever the number of sequences.  Causal with
+    different boundaries (queries that are the tail of a longer key sequence: chunked prefill,
+    decoding) aligns every sequence bottom-right on its own, which is not one offset of the packed
+    row: the rows then carry their own causal positions (varlen_positions, the qpos argument of the
+    operator).  Nothing is read back to the host.
     (No counterpart in the reference, which takes eq/ek directly, flash_triton.py:506.)"""
     assert q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be [total, heads, D]"
     same = cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q
-    if not same and causal:
-        same = cu_seqlens_k.shape == cu_seqlens_q.shape and bool(torch.equal(cu_seqlens_k, cu_seqlens_q))
-        if not same:
-            return _varlen_causal_by_sequence(q, k, v, cu_seqlens_q, cu_seqlens_k, sm_scale, window)
     Tq, H, _ = q.shape
     Tk = k.shape[0]
+    qpos = None
+    if not same:
+        assert cu_seqlens_q.shape == cu_seqlens_k.shape, "cu_seqlens_q and cu_seqlens_k must describe the same sequences"
+        if causal:
+            qpos = varlen_positions(cu_seqlens_q, cu_seqlens_k, Tq).view(1, Tq)
     eq = varlen_ids(cu_seqlens_q, Tq)
     ek = eq if (same and Tk == Tq) else varlen_ids(cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k, Tk)
     q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (q, k, v))
     out = attention(q4, k4, v4, causal, sm_scale, eq.view(1, 1, Tq).expand(1, H, Tq), ek.view(1, 1, Tk).expand(1, H, Tk),
-                    SCORE_FUNC_MODE1_DOC, window=window)
+                    SCORE_FUNC_MODE1_DOC, window=window, qpos=qpos)
     return out.squeeze(0).transpose(0, 1)
 
 
-def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda", window=0, prefix=0):
+def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_MODE0_NOPE, device="cuda", window=0, prefix=0,
+              qpos=None):
     """keep(i, j) as a bool tensor [B, H, M, N], evaluated by the device mask routine."""
     L = _cabi.lib()
     device = torch.device(device)
@@ -390,6 +399,10 @@ def mask_dump(B, H, M, N, causal, eq=None, ek=None, score_func_mode=SCORE_FUNC_M
             ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
             p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
             keep += [eq, ek, ws]
+            if qpos is not None:
+                qpos = qpos.to(device).to(torch.int32).contiguous()
+                p.qpos, p.qpos_stride = qpos.data_ptr(), (qpos.stride(0) if qpos.shape[0] > 1 else 0)
+                keep += [qpos]
             _cabi.check(L.fa_mask_plan(ctypes.byref(p), _stream_ptr(device)), "fa_mask_plan")
         out = torch.empty((B, H, M, N), dtype=torch.uint8, device=device)
         _cabi.check(L.fa_mask_dump(ctypes.byref(p), out.data_ptr(), _stream_ptr(device)), "fa_mask_dump")
