@@ -738,6 +738,21 @@ def test_fp32_tensors(case):
     _run_case(B, H, Hk, M, N, D, torch.float32, causal, doc, seed=5, tol_o=TOL_F32, tol_lse=TOL_F32)
 
 
+@pytest.mark.parametrize("M,N,D,window,kind", [(300, 300, 64, 0, "random"), (333, 77, 128, 0, "random"), (700, 900, 128, 40, "steps"),
+                                              (130, 190, 16, 7, "random"), (1300, 1300, 32, 0, "steps")])
+def test_fp32_per_row_causal_positions(M, N, D, window, kind):
+    """fp32 kernels with ids walk the permuted order of the plan and take the rows' diagonals from it."""
+    _run_case(1, 2, 1, M, N, D, torch.float32, True, True, seed=8 + M, window=window, qpos=kind, tol_o=TOL_F32, tol_lse=TOL_F32)
+
+
+def test_fp32_packed_documents_multi_tile():
+    """fp32 with ids over several 128-row tiles per group (local tiles, a padded boundary, global tiles),
+    per-head ids and grouped heads; causal and not."""
+    _run_case(1, 4, 2, 1100, 1100, 64, torch.float32, True, True, seed=31, tol_o=TOL_F32, tol_lse=TOL_F32)
+    _run_case(2, 2, 2, 700, 1000, 128, torch.float32, False, True, seed=32, per_head_ids=True, tol_o=TOL_F32, tol_lse=TOL_F32)
+    _run_case(1, 2, 2, 900, 900, 32, torch.float32, True, True, seed=33, ids_kind="alllocal", tol_o=TOL_F32, tol_lse=TOL_F32)
+
+
 def test_fp32_all_global_and_all_local_ids():
     _run_case(1, 2, 2, 160, 160, 64, torch.float32, True, True, seed=6, ids_kind="allglobal", tol_o=TOL_F32, tol_lse=TOL_F32)
     _run_case(1, 2, 2, 160, 160, 64, torch.float32, False, True, seed=6, ids_kind="alllocal", tol_o=TOL_F32, tol_lse=TOL_F32)
@@ -881,6 +896,35 @@ def test_varlen_fp32():
             for name, got, ref in (("o", out.detach(), ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
                 err = (sl(got.float().cpu()) - ref).abs().max().item()
                 assert err <= TOL_F32 * max(1.0, ref.abs().max().item()), f"sequence {s} {name} err {err}"
+
+
+def test_varlen_fp32_causal_with_longer_key_sequences():
+    """The one-launch causal packed batch with different boundaries on the fp32 kernels."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    lq, lk = [40, 3, 0, 100, 1, 200], [40, 200, 5, 164, 77, 333]
+    cuq = torch.tensor(np.concatenate([[0], np.cumsum(lq)]), dtype=torch.int32)
+    cuk = torch.tensor(np.concatenate([[0], np.cumsum(lk)]), dtype=torch.int32)
+    Tq, Tk, H, Hk, D = int(cuq[-1]), int(cuk[-1]), 2, 1, 64
+    g = torch.Generator().manual_seed(41)
+    q = torch.randn(Tq, H, D, generator=g); do = torch.randn(Tq, H, D, generator=g)
+    k = torch.randn(Tk, Hk, D, generator=g); v = torch.randn(Tk, Hk, D, generator=g)
+    print("varlen fp32 causal, longer key sequences", flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cuq.cuda(), cuk.cuda(), causal=True)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for s in range(len(lq)):
+        a, b, c, d = int(cuq[s]), int(cuq[s + 1]), int(cuk[s]), int(cuk[s + 1])
+        if a == b:
+            assert kd.grad[c:d].abs().max().item() == 0 and vd.grad[c:d].abs().max().item() == 0
+            continue
+        sq = lambda t: t[a:b].transpose(0, 1)[None]
+        sk = lambda t: t[c:d].transpose(0, 1)[None]
+        ro, _, rdq, rdk, rdv = O.attention_autograd(sq(q), sk(k), sk(v), sq(do), True, None, None, None, 0)
+        for name, got, ref, sl in (("o", out.detach(), ro, sq), ("dq", qd.grad, rdq, sq), ("dk", kd.grad, rdk, sk), ("dv", vd.grad, rdv, sk)):
+            err = (sl(got.float().cpu()) - ref).abs().max().item()
+            assert err <= TOL_F32 * max(1.0, ref.abs().max().item()), f"sequence {s} {name} err {err}"
 
 
 @pytest.mark.parametrize("D", [16, 128])

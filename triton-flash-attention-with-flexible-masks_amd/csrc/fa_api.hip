@@ -69,7 +69,6 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->workspace_bytes < fa_workspace_bytes(p)) return FA_ERR_WORKSPACE;
   }
   if (stage == 2) return FA_OK;
-  if (p->qpos != nullptr && p->dtype == FA_DTYPE_FP32) return FA_ERR_NOT_IMPLEMENTED;
   int rc;
   if ((rc = check_tensor(p->q, p->q_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
   if ((rc = check_tensor(p->k, p->k_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
@@ -123,7 +122,6 @@ static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratch
   a.eq_bs = a.eq_hs = a.ek_bs = a.ek_hs = a.pm_bs = a.pm_hs = a.qh_bs = a.qh_hs = 0;
   a.qs_bs = a.qs_hs = a.ks_bs = a.ks_hs = 0;
   a.nQs = a.nKs = a.Pp = 0;
-  a.qk_same = 0;
   a.dq_delta = (p->flags & FA_FLAG_DQ_DELTA) != 0;
   a.pair_spin = (p->flags & FA_FLAG_DEBUG_NO_PAIR_WAIT) ? 0 : kPairSpinDefault;
   a.bmask = nullptr; a.bm_bs = a.bm_hs = a.bm_rs = 0;
@@ -150,8 +148,6 @@ static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratch
     a.qs_bs = int64_t(w.Hq1) * w.nQs; a.qs_hs = w.Hq1 == 1 ? 0 : w.nQs;
     a.ks_bs = int64_t(w.Hk1) * w.nKs; a.ks_hs = w.Hk1 == 1 ? 0 : w.nKs;
     a.nQs = w.nQs; a.nKs = w.nKs; a.Pp = w.Pp;
-    a.qk_same = (p->eq == p->ek && p->M == p->N && p->eq_stride[0] == p->ek_stride[0] && p->eq_stride[1] == p->ek_stride[1] &&
-                 p->eq_stride[2] == p->ek_stride[2]) ? 1 : 0;
     const SplitCfg sc = w.split;
     a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);

@@ -282,7 +282,6 @@ struct KArgs {
   const unsigned char* bmask;
   int64_t bm_bs, bm_hs, bm_rs;
   int nBr, nBc;
-  int qk_same;            // eq and ek are one id vector (same pointer, strides and length): ksum also describes the rows
   float scale;            // sm_scale
   float scale_log2e;      // sm_scale * log2(e)
 };

@@ -17,11 +17,13 @@
 // rows 8*q4 + 4*(lane/32) + t; P^T / dS^T / P / dS are consumed as the B operand of the next
 // product straight from those registers (the contraction index is walked in that same order on
 // the A side), so nothing is exchanged or transposed.
-// Masks: rows are walked in natural order; the element masks are the routines of the 16-bit
-// kernels (same accumulator layout); a wave skips a 32x32 block when the causal bound or the id
-// intervals of its rows and of the block's keys (reduced from the ids staged with the tile)
-// exclude every pair.  With ids the int32 id copies of the mask plan are used (fa_mask_plan
-// must have run, as for the other types).
+// Masks: the element masks are the routines of the 16-bit kernels (same accumulator layout); a wave
+// skips a 32x32 block when the causal bound or the id intervals of its rows and of the block's keys
+// (reduced from the ids staged with the tile) exclude every pair.  Without ids rows are walked in
+// natural order.  With ids the query side is walked in the permuted order of the mask plan (local
+// rows first, then global rows: a tile of local rows meets the keys of its own documents only),
+// rows are gathered through the permutation, causal terms use the diagonal positions the plan
+// stored, and tiles that the plan's summaries rule out for the whole workgroup are not loaded.
 #include "fa_tile.h"
 
 namespace fa {
@@ -46,6 +48,21 @@ struct TileRegs {
       const bool ok = idx < N4 && row0 + r < nrows;
       const f32x4 z = {0.f, 0.f, 0.f, 0.f};
       v[i] = ok ? *reinterpret_cast<const f32x4*>(base + int64_t(row0 + r) * rs + 4 * c4) : z;
+    }
+  }
+  // the same for a tile whose rows are rows[0..31] of the matrix (-1: no row, reads as zero)
+  FA_DEV void load_rows(const float* base, int64_t rs, const int* rows) {
+    int ri[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + kThreads * i;
+      ri[i] = idx < N4 ? rows[idx / C4] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c4 = (threadIdx.x + kThreads * i) % C4;
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      v[i] = ri[i] >= 0 ? *reinterpret_cast<const f32x4*>(base + int64_t(ri[i]) * rs + 4 * c4) : z;
     }
   }
   FA_DEV void store(float* lds) const {
@@ -111,6 +128,73 @@ FA_DEV void wg_reduce3(int& lo, int& hi, int& glob) {
 template <int D>
 constexpr size_t lds_bytes() { return size_t(2 * kRows * (D + 1) + 4 * kRows + 64) * 4; }
 
+// Query side of the forward and dq kernels: which row a lane owns, its id, its causal limits, what
+// its wave and its workgroup can see.  Without ids: natural order.  With ids: tile `tile` of the
+// permuted order of the mask plan; the diagonal of a row sits at the position the plan stored.
+template <bool CAUSAL, bool DOC>
+struct QSideF32 {
+  int row, rowc;        // the lane's row (-1: none), clamped for loads
+  bool live;
+  int eq_i;
+  bool glob_i;
+  int lim_i, low_i;     // last / first key the row may see
+  int w_lim, w_low;     // largest last key / smallest first key among the wave's rows
+  bool w_any;           // the wave holds a row
+  int w_lo, w_hi, w_glob;
+  int g_lo, g_hi, g_glob;
+  int kt0, nkt;         // key tiles (of kRows) the workgroup walks: [kt0, nkt)
+  // returns false when the tile holds no row at all (uniform over the workgroup)
+  FA_DEV bool init(const KArgs& a, int b, int h, int tile, int wave, int lq) {
+    int posc, g_pmin, g_pmax, kfirst = 0, klast = 0x3fffffff;
+    if (!DOC) {
+      const int m0 = tile * 128, mw = m0 + wave * 32;
+      row = mw + lq < a.M ? mw + lq : -1;
+      posc = a.gap + min(mw + lq, a.M - 1);
+      eq_i = 0;
+      g_pmin = a.gap + m0; g_pmax = a.gap + min(m0 + 127, a.M - 1);
+    } else {
+      const IdSummary* qs = a.qsum + b * a.qs_bs + h * a.qs_hs + 2 * tile;
+      const IdSummary s0 = qs[0], s1 = qs[1];
+      const int64_t pi = b * a.pm_bs + h * a.pm_hs + tile * 128 + wave * 32 + lq;
+      row = a.perm[pi];
+      eq_i = a.peq[pi];
+      posc = a.ppos[pi];
+      if (s0.nvalid + s1.nvalid == 0) return false;
+      g_pmin = min(s0.rmin, s1.rmin); g_pmax = max(s0.rmax, s1.rmax);
+      kfirst = min(s0.kfirst, s1.kfirst); klast = max(s0.klast, s1.klast);
+    }
+    live = row >= 0;
+    rowc = live ? row : 0;
+    if (!live) posc = -1;
+    glob_i = eq_i >= 0;
+    lim_i = CAUSAL ? min(max(posc, a.pfx_m1), a.N - 1) : a.N - 1;
+    low_i = CAUSAL ? posc - a.win + 1 : -0x3fffffff;
+    w_any = __builtin_amdgcn_ballot_w64(live) != 0;
+    w_lim = half_max(live ? lim_i : -1);
+    w_low = half_min(live ? low_i : 0x7fffffff);
+    w_lo = 0x7fffffff; w_hi = (int)0x80000000; w_glob = 0;
+    if (DOC) {
+      w_lo = half_min(live && !glob_i ? eq_i : 0x7fffffff);
+      w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
+      w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
+    }
+    g_lo = w_lo; g_hi = w_hi; g_glob = w_glob;
+    if (DOC) wg_reduce3(g_lo, g_hi, g_glob);
+    const int n_end = CAUSAL ? min(a.N, max(g_pmax, a.pfx_m1) + 1) : a.N;
+    kt0 = CAUSAL ? max(0, g_pmin - a.win + 1) / kRows : 0;   // sliding window: first tile any row sees
+    nkt = (n_end + kRows - 1) / kRows;                       // the same for all waves: the tile stream has barriers
+    if (DOC) {                                               // the plan's key range of these rows (tiles of kSumRows keys)
+      if (klast < kfirst) nkt = 0;
+      else {
+        kt0 = max(kt0, kfirst * (kSumRows / kRows));
+        nkt = min(nkt, (klast + 1) * (kSumRows / kRows));
+      }
+    }
+    return true;
+  }
+  FA_DEV bool skips(int n0) const { return !w_any || n0 > w_lim || n0 + kRows - 1 < w_low; }
+};
+
 // ---------------------------------------------------------------------------------------------
 template <int D, bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
@@ -124,11 +208,12 @@ void fwd_f32_kernel(const KArgs a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lq = lane & 31, g = lane >> 5;
   const int BH = a.B * a.H;
-  const int nQt = (a.M + 127) / 128;
-  const int tile = nQt - 1 - blockIdx.x / BH;   // the last rows see the most keys: first
+  const int nQt = DOC ? a.Pp / 128 : (a.M + 127) / 128;
+  const int tile = nQt - 1 - blockIdx.x / BH;   // the last rows see the most keys (with ids: the global rows): first
   const int bh = blockIdx.x % BH, b = bh / a.H, h = bh % a.H, hk = h / a.G;
-  const int m0 = tile * 128, mw = m0 + wave * 32;
-  const int row = mw + lq, rowc = min(row, a.M - 1);
+  QSideF32<CAUSAL, DOC> qc;
+  if (!qc.init(a, b, h, tile, wave, lq)) return;
+  const int row = qc.row, rowc = qc.rowc;
 
   const float* qp = reinterpret_cast<const float*>(a.q) + b * a.q_bs + h * a.q_hs + int64_t(rowc) * a.q_rs;
   const float* kp = reinterpret_cast<const float*>(a.k) + b * a.k_bs + hk * a.k_hs;
@@ -144,24 +229,11 @@ void fwd_f32_kernel(const KArgs a) {
 #pragma unroll
     for (int s = 0; s < KS2; ++s) qreg[s] = -qreg[s];
   }
-  const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
-  const bool glob_i = eq_i >= 0;
-  const int lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;   // last key this row may see
-  const int low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;                 // first one (sliding window)
-  // the wave's rows: largest such limit, id interval of the local rows, any global row
-  const int w_last = min(mw + 31, a.M - 1);
-  const int w_lim = CAUSAL ? min(max(a.gap + w_last, a.pfx_m1), a.N - 1) : a.N - 1;
-  const int w_low = CAUSAL ? a.gap + mw - a.win + 1 : -0x3fffffff;   // smallest first key among the wave's rows
-  int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
-  if (DOC) {
-    const bool live = row < a.M;
-    w_lo = half_min(live && !glob_i ? eq_i : 0x7fffffff);
-    w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
-    w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
-  }
-  const int n_end = CAUSAL ? min(a.N, max(a.gap + min(m0 + 127, a.M - 1), a.pfx_m1) + 1) : a.N;
-  const int kt0 = CAUSAL ? max(0, a.gap + m0 - a.win + 1) / kRows : 0;   // sliding window: first tile any row sees
-  const int nkt = (n_end + kRows - 1) / kRows;   // the same for all waves: the tile stream has barriers
+  const int eq_i = qc.eq_i;
+  const bool glob_i = qc.glob_i;
+  const int lim_i = qc.lim_i, low_i = qc.low_i;
+  const int w_lo = qc.w_lo, w_hi = qc.w_hi, w_glob = qc.w_glob;
+  const int kt0 = qc.kt0, nkt = qc.nkt;
 
   f32x16 o[DBN];
 #pragma unroll
@@ -174,12 +246,8 @@ void fwd_f32_kernel(const KArgs a) {
   int rid = 0;
   // With ids, key tiles that no row of the workgroup can see (by the 64-key summaries of the mask
   // plan) are not even loaded: a packed batch costs its block diagonal, not the whole triangle.
-  int g_lo = w_lo, g_hi = w_hi, g_glob = w_glob;
-  const IdSummary* ksum = nullptr;
-  if (DOC) {
-    wg_reduce3(g_lo, g_hi, g_glob);
-    ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
-  }
+  const int g_lo = qc.g_lo, g_hi = qc.g_hi, g_glob = qc.g_glob;
+  const IdSummary* ksum = DOC ? a.ksum + b * a.ks_bs + h * a.ks_hs : nullptr;
   // block mask: the byte rows of the workgroup's two 64-row halves (the second one may lie past the last row)
   const unsigned char* bm0 = nullptr;
   const unsigned char* bm1 = nullptr;
@@ -224,7 +292,7 @@ void fwd_f32_kernel(const KArgs a) {
       if (DOC && threadIdx.x < kRows) rid = ekp[min(kt_next * kRows + (int)threadIdx.x, a.N - 1)];
     }
     kt = kt_next;
-    bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
+    bool skip = qc.skips(n0);
     if (!DOC && bm0 != nullptr && !skip) {   // the wave's 32 rows and the tile's 32 keys lie inside one block
       const unsigned char* r = wave >= 2 ? bm1 : bm0;
       skip = r == nullptr || r[n0 / FA_MASK_BLOCK] == 0;
@@ -275,7 +343,7 @@ void fwd_f32_kernel(const KArgs a) {
 
   const float l_tot = xhalf_sum(l_run);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  if (row < a.M) {
+  if (row >= 0) {
     float* op = reinterpret_cast<float*>(a.o) + b * a.o_bs + h * a.o_hs + int64_t(row) * a.o_rs;
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
@@ -303,11 +371,12 @@ void dq_f32_kernel(const KArgs a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lq = lane & 31, g = lane >> 5;
   const int BH = a.B * a.H;
-  const int nQt = (a.M + 127) / 128;
+  const int nQt = DOC ? a.Pp / 128 : (a.M + 127) / 128;
   const int tile = nQt - 1 - blockIdx.x / BH;
   const int bh = blockIdx.x % BH, b = bh / a.H, h = bh % a.H, hk = h / a.G;
-  const int m0 = tile * 128, mw = m0 + wave * 32;
-  const int row = mw + lq, rowc = min(row, a.M - 1);
+  QSideF32<CAUSAL, DOC> qc;
+  if (!qc.init(a, b, h, tile, wave, lq)) return;
+  const int row = qc.row, rowc = qc.rowc;
 
   const float* qp = reinterpret_cast<const float*>(a.q) + b * a.q_bs + h * a.q_hs + int64_t(rowc) * a.q_rs;
   const float* dop = reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs + int64_t(rowc) * a.do_rs;
@@ -328,27 +397,15 @@ void dq_f32_kernel(const KArgs a) {
 #pragma unroll
     for (int s = 0; s < KS2; ++s) part += op[2 * s + g] * doreg[s];
     delta_i = xhalf_sum(part);
-    if (row < a.M && g == 0) a.delta[(int64_t(b) * a.H + h) * a.M + row] = delta_i;
+    if (row >= 0 && g == 0) a.delta[(int64_t(b) * a.H + h) * a.M + row] = delta_i;
   } else {
     delta_i = a.delta[(int64_t(b) * a.H + h) * a.M + rowc];
   }
-  const int eq_i = DOC ? a.eq32[b * a.eq_bs + h * a.eq_hs + rowc] : 0;
-  const bool glob_i = eq_i >= 0;
-  const int lim_i = CAUSAL ? min(max(a.gap + rowc, a.pfx_m1), a.N - 1) : a.N - 1;
-  const int low_i = CAUSAL ? a.gap + rowc - a.win + 1 : -0x3fffffff;
-  const int w_last = min(mw + 31, a.M - 1);
-  const int w_lim = CAUSAL ? min(max(a.gap + w_last, a.pfx_m1), a.N - 1) : a.N - 1;
-  const int w_low = CAUSAL ? a.gap + mw - a.win + 1 : -0x3fffffff;   // smallest first key among the wave's rows
-  int w_lo = 0x7fffffff, w_hi = (int)0x80000000, w_glob = 0;
-  if (DOC) {
-    const bool live = row < a.M;
-    w_lo = half_min(live && !glob_i ? eq_i : 0x7fffffff);
-    w_hi = half_max(live && !glob_i ? eq_i : (int)0x80000000);
-    w_glob = __builtin_amdgcn_ballot_w64(live && glob_i) != 0;
-  }
-  const int n_end = CAUSAL ? min(a.N, max(a.gap + min(m0 + 127, a.M - 1), a.pfx_m1) + 1) : a.N;
-  const int kt0 = CAUSAL ? max(0, a.gap + m0 - a.win + 1) / kRows : 0;   // sliding window: first tile any row sees
-  const int nkt = (n_end + kRows - 1) / kRows;
+  const int eq_i = qc.eq_i;
+  const bool glob_i = qc.glob_i;
+  const int lim_i = qc.lim_i, low_i = qc.low_i;
+  const int w_lo = qc.w_lo, w_hi = qc.w_hi, w_glob = qc.w_glob;
+  const int kt0 = qc.kt0, nkt = qc.nkt;
 
   f32x16 acc[DBN];
 #pragma unroll
@@ -360,12 +417,8 @@ void dq_f32_kernel(const KArgs a) {
   int rid = 0;
   // With ids, key tiles that no row of the workgroup can see (by the 64-key summaries of the mask
   // plan) are not even loaded: a packed batch costs its block diagonal, not the whole triangle.
-  int g_lo = w_lo, g_hi = w_hi, g_glob = w_glob;
-  const IdSummary* ksum = nullptr;
-  if (DOC) {
-    wg_reduce3(g_lo, g_hi, g_glob);
-    ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
-  }
+  const int g_lo = qc.g_lo, g_hi = qc.g_hi, g_glob = qc.g_glob;
+  const IdSummary* ksum = DOC ? a.ksum + b * a.ks_bs + h * a.ks_hs : nullptr;
   // block mask: the byte rows of the workgroup's two 64-row halves (the second one may lie past the last row)
   const unsigned char* bm0 = nullptr;
   const unsigned char* bm1 = nullptr;
@@ -410,7 +463,7 @@ void dq_f32_kernel(const KArgs a) {
       if (DOC && threadIdx.x < kRows) rid = ekp[min(kt_next * kRows + (int)threadIdx.x, a.N - 1)];
     }
     kt = kt_next;
-    bool skip = mw >= a.M || n0 > w_lim || n0 + kRows - 1 < w_low;
+    bool skip = qc.skips(n0);
     if (!DOC && bm0 != nullptr && !skip) {   // the wave's 32 rows and the tile's 32 keys lie inside one block
       const unsigned char* r = wave >= 2 ? bm1 : bm0;
       skip = r == nullptr || r[n0 / FA_MASK_BLOCK] == 0;
@@ -446,7 +499,7 @@ void dq_f32_kernel(const KArgs a) {
         [&](int i, float x) __attribute__((always_inline)) { acc[i / 16] = mfma_f32(x, s[i % 16], acc[i / 16]); });
   }
 
-  if (row < a.M) {
+  if (row >= 0) {
     float* dqp = reinterpret_cast<float*>(a.dq) + b * a.dq_bs + h * a.dq_hs + int64_t(row) * a.dq_rs;
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
@@ -469,8 +522,9 @@ void dkdv_f32_kernel(const KArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* lqt = reinterpret_cast<float*>(smem);
   float* ldo = lqt + kRows * RS;
-  float* laux = ldo + kRows * RS;               // [LSE | delta | eq] x 32
+  float* laux = ldo + kRows * RS;               // [LSE | delta | eq | row name] x 32
   const int* leq = reinterpret_cast<const int*>(laux + 2 * kRows);
+  const int* lnm = reinterpret_cast<const int*>(laux + 3 * kRows);
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lq = lane & 31, g = lane >> 5;
@@ -486,14 +540,19 @@ void dkdv_f32_kernel(const KArgs a) {
 #pragma unroll
   for (int s = 0; s < KS2; ++s) { kreg[s] = kp[2 * s + g]; vreg[s] = vp[2 * s + g]; }
   const float c = a.scale_log2e;
-  // rows that may see this lane's key: [row_lo, row_lo + row_span)
-  // (causal: from the diagonal on, or from row 0 for a key of the prefix; sliding window: `win` rows)
-  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - a.gap)) : 0;
-  const int row_hi = CAUSAL ? min(a.M - 1, key - a.gap + a.win - 1) : a.M - 1;
+  // A row is named by its index (its diagonal sits at key gap + index) or, with ids, by the diagonal
+  // position the mask plan stored for it (offset 0, names up to kPosMax; -1: no row).
+  // Rows that may see this lane's key: names [row_lo, row_lo + row_span)
+  // (causal: from the diagonal on, or from 0 for a key of the prefix; sliding window: `win` names)
+  const int gk = DOC ? 0 : a.gap;
+  const int rcap = DOC ? kPosMax : a.M - 1;
+  const int row_lo = CAUSAL ? (key <= a.pfx_m1 ? 0 : max(0, key - gk)) : 0;
+  const int row_hi = CAUSAL ? min(rcap, key - gk + a.win - 1) : rcap;
   const unsigned row_span = (key < a.N && row_hi >= row_lo) ? (unsigned)(row_hi - row_lo + 1) : 0u;
-  const int mt0 = CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - a.gap) / kRows) : 0;
-  const int wg_rhi = CAUSAL ? min(a.M - 1, n0 + 127 - a.gap + a.win - 1) : a.M - 1;   // last row that sees a key of the workgroup
-  const int nMt = max(0, wg_rhi + kRows) / kRows;
+  const int wg_rhi = CAUSAL ? min(rcap, n0 + 127 - gk + a.win - 1) : rcap;   // last name that sees a key of the workgroup
+  // query tiles of 32 rows: natural order from the diagonal on, or every tile of the permuted order
+  const int mt0 = DOC ? 0 : (CAUSAL ? (n0 <= a.pfx_m1 ? 0 : max(0, n0 - gk) / kRows) : 0);
+  const int nMt = DOC ? a.Pp / kRows : max(0, wg_rhi + kRows) / kRows;
 
   f32x16 dv[DBN], dk[DBN];
 #pragma unroll
@@ -507,38 +566,48 @@ void dkdv_f32_kernel(const KArgs a) {
     const float* dop = reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs;
     const float* lsep = a.lse + (int64_t(b) * a.H + h) * a.M;
     const float* delp = a.delta + (int64_t(b) * a.H + h) * a.M;
-    const int* eqp = DOC ? a.eq32 + b * a.eq_bs + h * a.eq_hs : nullptr;
+    const int* pmp = DOC ? a.perm + b * a.pm_bs + h * a.pm_hs : nullptr;
+    const int* pqp = DOC ? a.peq + b * a.pm_bs + h * a.pm_hs : nullptr;
+    const int* ppp = DOC ? a.ppos + b * a.pm_bs + h * a.pm_hs : nullptr;
     int ek_j = 0, wk_lo = 0, wk_hi = 0;
     if (DOC) {
       ek_j = a.ek32[b * a.ek_bs + h * a.ek_hs + keyc];
       wk_lo = half_min(key < a.N ? ek_j : 0x7fffffff);
       wk_hi = half_max(key < a.N ? ek_j : (int)0x80000000);
     }
-    // one auxiliary value per thread of the first three groups of 32: LSE, delta, eq of a tile row
-    auto aux_load = [&](int m0) -> float {
-      const int r = min(m0 + (int)(threadIdx.x & 31), a.M - 1);
-      const int which = threadIdx.x >> 5;
-      if (which == 0) return lsep[r];
-      if (which == 1) return delp[r];
-      if (which == 2 && DOC) return __int_as_float(eqp[r]);
-      return 0.f;
+    // one auxiliary value per thread of the first four groups of 32: LSE, delta, id, name of a tile row
+    auto aux_load = [&](int mt) -> float {
+      const int t = threadIdx.x & 31, which = threadIdx.x >> 5;
+      if (!DOC) {
+        const int r = mt * kRows + t, rc = min(r, a.M - 1);
+        if (which == 0) return lsep[rc];
+        if (which == 1) return delp[rc];
+        if (which == 3) return __int_as_float(r < a.M ? r : -1);
+        return 0.f;
+      }
+      if (which == 2) return __int_as_float(pqp[mt * kRows + t]);
+      if (which == 3) return __int_as_float(ppp[mt * kRows + t]);
+      const int r = max(pmp[mt * kRows + t], 0);
+      return which == 0 ? lsep[r] : delp[r];
     };
-    // When eq and ek are one id vector (self-attention), the 64-key summaries of the plan describe
-    // the query rows as well: query tiles that no key of the workgroup can meet are not even loaded.
+    // With ids: query tiles whose 64-entry summary of the plan excludes every key of the workgroup
+    // (no row, ids that cannot meet, diagonals before the first key or beyond the window) are not loaded.
     int gk_lo = wk_lo, gk_hi = wk_hi, gk_unused = 0;
-    const IdSummary* rsum = nullptr;
-    if (DOC && a.qk_same) {
+    const IdSummary* qsum = nullptr;
+    if (DOC) {
       wg_reduce3(gk_lo, gk_hi, gk_unused);
-      rsum = a.ksum + b * a.ks_bs + h * a.ks_hs;
+      qsum = a.qsum + b * a.qs_bs + h * a.qs_hs;
     }
     // block mask: the one or two byte columns of the workgroup's 128 keys
     const unsigned char* bmc = (!DOC && a.bmask != nullptr) ? a.bmask + b * a.bm_bs + h * a.bm_hs + n0 / FA_MASK_BLOCK : nullptr;
     const bool bm_two = n0 / FA_MASK_BLOCK + 1 < a.nBc;
     auto next_mt = [&](int mt) {
-      if (DOC && rsum != nullptr)
+      if (DOC)
         while (mt < nMt) {
-          const IdSummary qs = rsum[(mt * kRows) / kSumRows];   // ids of 64 rows: any id >= 0 is a global row
-          if (doc_may_keep(qs.lo, qs.hi, qs.hi >= 0, gk_lo, gk_hi)) break;
+          const IdSummary qs = qsum[(mt * kRows) / kSumRows];
+          const bool out = qs.nvalid == 0 || !doc_may_keep(qs.lo, qs.hi, qs.glob, gk_lo, gk_hi) ||
+                           (CAUSAL && ((qs.rmax < n0 && n0 > a.pfx_m1) || qs.rmin > wg_rhi));
+          if (!out) break;
           ++mt;
         }
       if (bmc != nullptr)
@@ -551,32 +620,36 @@ void dkdv_f32_kernel(const KArgs a) {
     };
     TileRegs<D> rq, rdo;
     float raux = 0.f;
+    auto load_tile = [&](int mt) {
+      if (DOC) {
+        rq.load_rows(qp, a.q_rs, pmp + mt * kRows);
+        rdo.load_rows(dop, a.do_rs, pmp + mt * kRows);
+      } else {
+        rq.load(qp, a.q_rs, mt * kRows, a.M);
+        rdo.load(dop, a.do_rs, mt * kRows, a.M);
+      }
+      if (threadIdx.x < 4 * kRows) raux = aux_load(mt);
+    };
     int mt = next_mt(mt0);
-    if (mt < nMt) {
-      rq.load(qp, a.q_rs, mt * kRows, a.M);
-      rdo.load(dop, a.do_rs, mt * kRows, a.M);
-      if (threadIdx.x < 3 * kRows) raux = aux_load(mt * kRows);
-    }
+    if (mt < nMt) load_tile(mt);
     while (mt < nMt) {
-      const int m0 = mt * kRows;
       const int mt_next = next_mt(mt + 1);
       __syncthreads();
       rq.store(lqt);
       rdo.store(ldo);
-      if (threadIdx.x < 3 * kRows) laux[threadIdx.x] = raux;
+      if (threadIdx.x < 4 * kRows) laux[threadIdx.x] = raux;
       __syncthreads();
-      if (mt_next < nMt) {
-        rq.load(qp, a.q_rs, mt_next * kRows, a.M);
-        rdo.load(dop, a.do_rs, mt_next * kRows, a.M);
-        if (threadIdx.x < 3 * kRows) raux = aux_load(mt_next * kRows);
-      }
+      if (mt_next < nMt) load_tile(mt_next);
       mt = mt_next;
-      bool skip = nw >= a.N || (CAUSAL && ((a.gap + min(m0 + kRows - 1, a.M - 1) < nw && nw > a.pfx_m1) ||
-                                           a.gap + m0 - a.win + 1 > nw + 31));
+      // names of the tile's rows (-1: none): smallest / largest among the 32
+      const int nm = lnm[lq];
+      const int t_min = half_min(nm >= 0 ? nm : 0x7fffffff), t_max = half_max(nm);
+      bool skip = nw >= a.N || t_max < 0 ||
+                  (CAUSAL && ((gk + t_max < nw && nw > a.pfx_m1) || gk + t_min - a.win + 1 > nw + 31));
       if (bmc != nullptr && !skip)   // the wave's 32 keys and the tile's 32 rows lie inside one block
-        skip = bmc[int64_t(m0 / FA_MASK_BLOCK) * a.bm_rs + (wave >= 2 ? 1 : 0)] == 0;
+        skip = bmc[int64_t((t_min / FA_MASK_BLOCK)) * a.bm_rs + (wave >= 2 ? 1 : 0)] == 0;
       if (DOC && !skip) {
-        const bool rv_ = m0 + lq < a.M;
+        const bool rv_ = nm >= 0;
         const int id = leq[lq];
         const bool loc = rv_ && id < 0;
         const int q_lo = half_min(loc ? id : 0x7fffffff), q_hi = half_max(loc ? id : (int)0x80000000);
@@ -601,9 +674,10 @@ void dkdv_f32_kernel(const KArgs a) {
         const f32x4 Lv = *reinterpret_cast<const f32x4*>(laux + i0);
         const f32x4 dl = *reinterpret_cast<const f32x4*>(laux + kRows + i0);
         const i32x4 eqv = *reinterpret_cast<const i32x4*>(leq + i0);
+        const i32x4 nmv = *reinterpret_cast<const i32x4*>(lnm + i0);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          bool keep = (unsigned)(m0 + i0 + t - row_lo) < row_span;
+          bool keep = (unsigned)(nmv[t] - row_lo) < row_span;
           if (DOC) keep = keep && (eqv[t] >= 0 || eqv[t] == ek_j);
           const float p = fast_exp2(__builtin_fmaf(x[4 * q4 + t], c, -Lv[t]));
           x[4 * q4 + t] = keep ? p : 0.f;
@@ -668,7 +742,8 @@ template <int WHICH, int D, bool CAUSAL, bool DOC>
 int launch_one(const KArgs& a, hipStream_t s) {
   auto kern = WHICH == kFwd ? fwd_f32_kernel<D, CAUSAL, DOC> : WHICH == kDq ? dq_f32_kernel<D, CAUSAL, DOC>
                                                                             : dkdv_f32_kernel<D, CAUSAL, DOC>;
-  const int blocks = WHICH == kDkdv ? ((a.N + 127) / 128) * a.B * a.Hk : ((a.M + 127) / 128) * a.B * a.H;
+  // query tiles: of the natural order, or of the mask plan's permuted order with ids
+  const int blocks = WHICH == kDkdv ? ((a.N + 127) / 128) * a.B * a.Hk : (DOC ? a.Pp / 128 : (a.M + 127) / 128) * a.B * a.H;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds_bytes<D>(), lds_allowed)) return e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreads), lds_bytes<D>(), s, a);
