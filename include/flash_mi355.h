@@ -192,8 +192,8 @@ int fa_fwd(const fa_params* p, void* stream);
    FA_STATIC_WS_BYTES inside the library (held by every GPU the library runs on until the process
    ends).  The call enqueues the plan kernels and the forward on `stream` and allocates nothing, on
    the host or the device.  Problems whose plan does not fit the array are refused with
-   FA_ERR_WORKSPACE (the plan needs about 12 bytes per query row and 5 per key, times the batch, times
-   the heads unless the ids' head stride is 0; the headline shape B=1 H=32 L=16384 takes 0.4 MB plus
+   FA_ERR_WORKSPACE (the plan needs about 17 bytes per query row and 5 per key, times the batch, times
+   the heads unless the ids' head stride is 0; the headline shape B=1 H=32 L=16384 takes 0.5 MB plus
    split scratch).  Every call on a GPU uses that GPU's one array, which keeps the last call's
    contents: calls that overlap on one GPU (different streams, different threads) race and must be
    ordered by the caller; a backward needs its own fa_mask_plan into a caller's workspace.

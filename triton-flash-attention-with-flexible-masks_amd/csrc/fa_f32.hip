@@ -582,7 +582,6 @@ void dkdv_f32_kernel(const KArgs a) {
         const int r = mt * kRows + t, rc = min(r, a.M - 1);
         if (which == 0) return lsep[rc];
         if (which == 1) return delp[rc];
-        if (which == 3) return __int_as_float(r < a.M ? r : -1);
         return 0.f;
       }
       if (which == 2) return __int_as_float(pqp[mt * kRows + t]);
@@ -640,10 +639,12 @@ void dkdv_f32_kernel(const KArgs a) {
       if (threadIdx.x < 4 * kRows) laux[threadIdx.x] = raux;
       __syncthreads();
       if (mt_next < nMt) load_tile(mt_next);
+      const int m0 = mt * kRows;   // natural order only
       mt = mt_next;
       // names of the tile's rows (-1: none): smallest / largest among the 32
-      const int nm = lnm[lq];
-      const int t_min = half_min(nm >= 0 ? nm : 0x7fffffff), t_max = half_max(nm);
+      const int nm = DOC ? lnm[lq] : (m0 + lq < a.M ? m0 + lq : -1);
+      const int t_min = DOC ? half_min(nm >= 0 ? nm : 0x7fffffff) : m0;
+      const int t_max = DOC ? half_max(nm) : min(m0 + kRows - 1, a.M - 1);
       bool skip = nw >= a.N || t_max < 0 ||
                   (CAUSAL && ((gk + t_max < nw && nw > a.pfx_m1) || gk + t_min - a.win + 1 > nw + 31));
       if (bmc != nullptr && !skip)   // the wave's 32 keys and the tile's 32 rows lie inside one block
@@ -674,7 +675,8 @@ void dkdv_f32_kernel(const KArgs a) {
         const f32x4 Lv = *reinterpret_cast<const f32x4*>(laux + i0);
         const f32x4 dl = *reinterpret_cast<const f32x4*>(laux + kRows + i0);
         const i32x4 eqv = *reinterpret_cast<const i32x4*>(leq + i0);
-        const i32x4 nmv = *reinterpret_cast<const i32x4*>(lnm + i0);
+        i32x4 nmv = {m0 + i0, m0 + i0 + 1, m0 + i0 + 2, m0 + i0 + 3};   // rows past the end lie beyond every span
+        if (DOC) nmv = *reinterpret_cast<const i32x4*>(lnm + i0);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           bool keep = (unsigned)(nmv[t] - row_lo) < row_span;
