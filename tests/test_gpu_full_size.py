@@ -166,3 +166,40 @@ def test_cfg1_fp32_doc_causal_in_full():
     for nm, got, ref in (("o", out, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
         err = (got.detach().float().cpu() - ref).abs().max().item()
         assert err <= tol * max(1.0, ref.abs().max().item()), (nm, err)
+
+
+def test_packed_prefill_with_per_sequence_alignment_at_16k_keys():
+    """A packed causal batch at the headline key length whose sequences have more keys than queries
+    (chunked prefill: the queries are the tail of every sequence), one launch per kernel: ragged
+    sequence lengths, 8192 queries against 16384 keys, 8 heads over the 8 XCDs.  Properties over every
+    head (V = 1 => O = 1 wherever a row exists), and three sequences -- the first, a middle one and the
+    last -- against the oracle run on that sequence alone (the reference's rectangular causal case,
+    flash_triton.py:520-521)."""
+    from flash_mi355 import attention_varlen
+    from oracle import attention_oracle as O
+    rng = np.random.default_rng(5)
+    S = 12
+    lq = rng.multinomial(8192 - 16 * S, np.ones(S) / S) + 16
+    lk = lq + (rng.multinomial(8192 - 8 * S, np.ones(S) / S) + 8)
+    cq = np.concatenate([[0], np.cumsum(lq)]); ck = np.concatenate([[0], np.cumsum(lk)])
+    Tq, Tk, H, D = int(cq[-1]), int(ck[-1]), 8, 128
+    assert (Tq, Tk) == (8192, 16384)
+    g = torch.Generator().manual_seed(6)
+    q, do = (torch.randn(Tq, H, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    k, v = (torch.randn(Tk, H, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    print(f"case packed prefill lq={lq.tolist()} lk={lk.tolist()}", flush=True)
+    cuq, cuk = torch.from_numpy(cq).to(torch.int32).cuda(), torch.from_numpy(ck).to(torch.int32).cuda()
+    ones = attention_varlen(q.cuda(), k.cuda(), torch.ones_like(v).cuda(), cuq, cuk, causal=True)
+    assert torch.equal(ones, torch.ones_like(ones))
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = attention_varlen(qd, kd, vd, cuq, cuk, causal=True)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    for s in (0, S // 2, S - 1):
+        a, b, c, d = int(cq[s]), int(cq[s + 1]), int(ck[s]), int(ck[s + 1])
+        sq = lambda t: t[a:b].transpose(0, 1)[None]
+        sk = lambda t: t[c:d].transpose(0, 1)[None]
+        ro, _, rdq, rdk, rdv = O.attention_autograd(sq(q), sk(k), sk(v), sq(do), True, None, None, None, 0)
+        assert (sq(out.detach().float().cpu()) - ro).abs().max().item() <= TOL_O
+        for nm, got, ref, sl in (("dq", qd.grad, rdq, sq), ("dk", kd.grad, rdk, sk), ("dv", vd.grad, rdv, sk)):
+            check_close(f"sequence {s} {nm}", sl(got.float().cpu()), ref)
