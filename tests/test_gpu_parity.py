@@ -814,6 +814,23 @@ def test_window_needs_causal():
         attention(q, q, q, True, window=8, prefix=8)
 
 
+@pytest.mark.parametrize("seed", list(range(300, 324)))
+def test_random_shapes_with_per_row_positions(seed):
+    """Third seeded sweep: per-row causal positions (any order, or the steps of a packed batch) over the
+    three element types, all head sizes, more or fewer queries than keys, windows, id layouts."""
+    rng = np.random.default_rng(seed)
+    D = int(rng.choice([16, 32, 64, 128]))
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+    B = int(rng.integers(1, 3)); Hk = int(rng.integers(1, 3)); H = Hk * int(rng.integers(1, 3))
+    M = int(rng.integers(1, 700))
+    N = int(rng.integers(2000, 2600)) if rng.random() < 0.2 else int(rng.integers(1, 1500))
+    window = int(rng.choice([0, 0, 0, 5, 64, 300]))
+    f32 = dtype == torch.float32
+    _run_case(B, H, Hk, M, N, D, dtype, True, True, seed=seed, ids_kind=str(rng.choice(["uniform", "uniform", "allglobal", "alllocal"])),
+              per_head_ids=bool(rng.random() < 0.3), window=window, qpos=str(rng.choice(["random", "steps"])),
+              tol_o=TOL_F32 if f32 else TOL_O, tol_lse=TOL_F32 if f32 else TOL_LSE)
+
+
 @pytest.mark.parametrize("seed", list(range(200, 232)))
 def test_random_shapes_all_types_and_masks(seed):
     """Second seeded sweep: the three element types, and on causal draws a sliding window or a
