@@ -831,6 +831,19 @@ def test_random_shapes_with_per_row_positions(seed):
               tol_o=TOL_F32 if f32 else TOL_O, tol_lse=TOL_F32 if f32 else TOL_LSE)
 
 
+@pytest.mark.xfail(strict=False, reason="one element of dK lands 3 % over the per-element bound: a finding, kept visible")
+def test_case_found_outside_the_bound():
+    """Found by a sweep of about 1500 random cases outside this suite (identical before and after the
+    per-row-position work, so not a regression): grouped heads, bf16, local ids, window 876, M 243 against
+    N 1419.  One element of dK comes out as -3.1875 where the exact value is -3.2081: 0.0128 of error from the
+    16-bit storage of P and dS inside the kernel plus the output's own rounding (a bf16 step is 0.0156 there),
+    0.0206 in all against the bound of 0.02.  The CPU model of the storage roundings
+    (oracle.attention_grads(store_dtype=...)) with the output rounding on top stays at 0.76 of the bound on the
+    same inputs, so the kernel is somewhat worse than that model here.  Every other element of the case, and
+    every case of the suite, is inside the bound."""
+    _run_case(1, 4, 2, 243, 1419, 128, torch.bfloat16, True, True, seed=5012, ids_kind="alllocal", window=876)
+
+
 @pytest.mark.parametrize("seed", list(range(200, 232)))
 def test_random_shapes_all_types_and_masks(seed):
     """Second seeded sweep: the three element types, and on causal draws a sliding window or a
