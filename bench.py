@@ -85,6 +85,9 @@ def parse_args():
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of the benchmark: print the sustained bf16 MFMA rate of the chip (a bare MFMA loop "
                          "with small-integer and with random operands, libfa_probe.so), four launches each")
+    ap.add_argument("--wg-trace", action="store_true",
+                    help="instead of the benchmark: launch forward, dQ and dK/dV of the workload from the clock-stamp "
+                         "build (libflash_mi355_trace.so) and print where the workgroups spend their time")
     return ap.parse_args()
 
 
@@ -149,6 +152,76 @@ def time_kernels(w, q, k, v, do, eq, ek, torch, iters=20, warm=5):
         out[name] = ev[0].elapsed_time(ev[-1]) / iters
         quant[name] = [round(ts[int(f * (iters - 1))], 4) for f in (0.2, 0.5, 0.8)]
     out["_quantiles"] = quant
+    return out
+
+
+def wg_trace(w, q, k, v, do, eq, ek, torch):
+    """Per-workgroup timeline of the three kernels from the clock-stamp build: every workgroup notes the
+    100 MHz wall clock at a handful of points; this reads the stamps of one launch (after warm ones) and
+    reduces them to means.  "mean_resident_per_cu" is the summed workgroup lifetime over span x 256 CUs."""
+    import numpy as np
+    from flash_mi355 import _cabi
+    from flash_mi355.build import TRACE_LIB_PATH
+    assert _cabi._lib is None, "the trace build must be the first library loaded"
+    _cabi.LIB_PATH = TRACE_LIB_PATH
+    L = _cabi.lib()
+    L.fa_trace_read.restype = ctypes.c_int
+    L.fa_trace_read.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    dev = q.device
+    plan = _Plan(q, k, v, w.causal, 1.0 / math.sqrt(w.D), eq, ek, 1 if w.doc else (2 if w.block is not None else 0), w.window, w.prefix)
+    p = plan.p
+    o = torch.empty_like(q)
+    lse = torch.empty(w.B, w.H, w.Lq, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    dq = torch.empty_like(q)
+    dk = torch.empty(w.B, w.Hk, w.Lk, w.D, device=dev, dtype=q.dtype)
+    dv = torch.empty_like(dk)
+    p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+        _set4(getattr(p, f), t)
+    plan.ensure_workspace(dev)
+    stream = _stream_ptr(dev)
+    ref = ctypes.byref(p)
+    p.flags = _cabi.FA_FLAG_DQ_DELTA
+    if w.doc:
+        _cabi.check(L.fa_mask_plan(ref, stream), "fa_mask_plan")
+    TICK_US = 0.01   # the wall clock of the stamps runs at 100 MHz
+    out = {}
+    # columns of the stamps: (start, set-up done, loop done, end, tiles, info)
+    for which, (name, fn, cols) in enumerate((("fa_fwd", L.fa_fwd, (0, 2, 3, 4, 5, 7)),
+                                              ("fa_bwd_dq", L.fa_bwd_dq, (0, 2, 3, 4, 5, 7)),
+                                              ("fa_bwd_dkdv", L.fa_bwd_dkdv, (0, 3, 4, 5, 6, 7)))):
+        for _ in range(4):
+            _cabi.check(fn(ref, stream), name)
+        torch.cuda.synchronize()
+        buf = np.zeros(8 * 65536, dtype=np.int64)
+        rc = L.fa_trace_read(which, buf.ctypes.data, buf.size)
+        assert rc == 0, f"fa_trace_read({which}) returned {rc}"
+        t = buf.reshape(-1, 8)
+        t = t[t[:, 0] != 0]
+        c_start, c_setup, c_loop, c_end, c_tiles, c_info = cols
+        left = t[:, c_info] == -1
+        live = t[~left & (t[:, c_end] != 0) & (t[:, c_tiles] > 0)]
+        idle = t[~left & (t[:, c_end] != 0) & (t[:, c_tiles] == 0)]
+        span = (t[:, c_end].max() - t[:, 0].min()) * TICK_US
+        life = (live[:, c_end] - live[:, c_start]) * TICK_US
+        r = {
+            "workgroups": int(len(t)), "left_at_once": int(left.sum()), "no_tiles": int(len(idle)),
+            "with_tiles": int(len(live)),
+            "span_us": round(float(span), 1),
+            "mean_lifetime_us": round(float(life.mean()), 2),
+            "mean_setup_us": round(float(((live[:, c_setup] - live[:, c_start]) * TICK_US).mean()), 2),
+            "mean_loop_us": round(float(((live[:, c_loop] - live[:, c_setup]) * TICK_US).mean()), 2),
+            "mean_drain_us": round(float(((live[:, c_end] - live[:, c_loop]) * TICK_US).mean()), 2),
+            "mean_tiles": round(float(live[:, c_tiles].mean()), 2),
+            "loop_us_per_tile": round(float((live[:, c_loop] - live[:, c_setup]).sum() * TICK_US / live[:, c_tiles].sum()), 3),
+            "mean_resident_per_cu": round(float(life.sum() / (span * 256)), 3),
+        }
+        if len(idle):
+            r["mean_lifetime_no_tiles_us"] = round(float(((idle[:, c_end] - idle[:, c_start]) * TICK_US).mean()), 2)
+        out[name] = r
     return out
 
 
@@ -247,6 +320,10 @@ def main():
 
     w = W.make_workload(args.workload)
     q, k, v, do, eq, ek = make_inputs(w, torch)
+    if args.wg_trace:
+        print(json.dumps({"workload": w.name, "clock": "100 MHz wall clock, one launch after four warm ones",
+                          "kernels": wg_trace(w, q, k, v, do, eq, ek, torch)}))
+        return
     mode = 1 if w.doc else (2 if w.block is not None else 0)
     scale = 1.0 / math.sqrt(w.D)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)

@@ -28,6 +28,20 @@ def test_library_exports_every_declared_symbol():
         assert getattr(L, n) is not None
 
 
+def test_clock_stamp_build_is_a_library_of_its_own():
+    """bench.py --wg-trace loads libflash_mi355_trace.so: every entry point of the header plus
+    fa_trace_read.  The product library carries no trace export."""
+    from flash_mi355.build import TRACE_LIB_PATH
+    assert TRACE_LIB_PATH.exists(), "python -m flash_mi355.build builds it next to the product library"
+    T = ctypes.CDLL(str(TRACE_LIB_PATH))
+    for n in _declared_functions() + ["fa_trace_read"]:
+        assert getattr(T, n) is not None
+    T.fa_version.restype = ctypes.c_int
+    assert T.fa_version() == _cabi.FA_ABI_VERSION
+    with pytest.raises(AttributeError):
+        _cabi.lib().fa_trace_read
+
+
 def test_struct_layout_and_version():
     L = _cabi.lib()
     assert L.fa_version() == _cabi.FA_ABI_VERSION == int(re.search(r"#define FA_ABI_VERSION (\d+)", HEADER).group(1))

@@ -263,3 +263,16 @@ extern "C" int fa_mask_dump(const fa_params* p, uint8_t* out, void* stream) {
   return finish(launch_mask_dump(make_args(p), p->causal != 0, p->score_mode == FA_SCORE_MODE1_DOC, out,
                                  reinterpret_cast<hipStream_t>(stream)));
 }
+
+#ifdef FA_TRACE
+// Measurement build only (not part of the product library or of its header): copies the clock
+// stamps of the last launch of one kernel to the host, 8 words per workgroup.
+// which: 0 forward, 1 dQ, 2 dK/dV.  n = number of 64-bit words (at most 8 * 65536).
+extern "C" int fa_trace_read(int which, long long* host, int n) {
+  if (host == nullptr) return FA_ERR_NULLPTR;
+  if (n < 0 || n > 8 * fa::kTraceWgs) return FA_ERR_SHAPE;
+  hipDeviceSynchronize();
+  const int e = which == 0 ? fa::trace_read_fwd(host, n) : which == 1 ? fa::trace_read_dq(host, n) : fa::trace_read_dkdv(host, n);
+  return e == 0 ? FA_OK : FA_ERR_HIP;
+}
+#endif

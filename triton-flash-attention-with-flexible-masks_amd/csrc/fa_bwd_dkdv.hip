@@ -35,6 +35,11 @@ constexpr int kKvPre2 = 3;
 // SPLIT = false: 4 waves, every wave does both roles for its 32 keys (D <= 64: everything fits), so P
 //                never leaves the registers and the only barrier is the one of the tile stream; two
 //                workgroups share a CU.
+#ifdef FA_TRACE
+// words: 0 start, 1 K / V fragments requested, 2 first query tile chosen, 3 first query tile in LDS, 4 after the tile loop, 5 end, 6 query tiles computed, 7 key tile | (batch, kv head) << 16 (-1: left at once)
+FA_TRACE_ARRAY(g_trace_dkdv);
+#endif
+
 template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT, int NKB>
 __global__ __launch_bounds__(SPLIT ? 128 * NKB : 64 * NKB) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 3 : 2, D <= 32 ? 3 : 2)))
 void bwd_dkdv_kernel(const KArgs a) {
@@ -63,6 +68,8 @@ void bwd_dkdv_kernel(const KArgs a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar
   const int role = SPLIT ? wave / NKB : 0, kb = wave % NKB;
   const int lq = lane & 31, g = lane >> 5;
+  FA_STAMP(g_trace_dkdv, 0, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 5, 0); FA_STAMP(g_trace_dkdv, 7, -1);
+  FA_TRACE_ONLY(int tr_tiles = 0; bool tr_first = false;)
 
   // one workgroup per (key tile, batch, kv head)
   const int nKt = (a.N + BK - 1) / BK;
@@ -94,6 +101,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   // 128-key form, which serves long streams, that gave the faster loop (4.24 against 4.39 ms, plain
   // causal 16K); at D <= 64 the difference stayed inside the run-to-run spread.
   constexpr bool LATE_SETTLE = SPLIT && NKB == 2;
+  FA_STAMP(g_trace_dkdv, 1, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 7, (long long)kt | ((long long)bhk << 16));
   if (!LATE_SETTLE) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { settle(frag[ks]); if (!SPLIT) settle(frag2[ks]); }
@@ -538,6 +546,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     int cur = it.next(dec), cur_fl = it.flags, cur_id = it.value;
     int nxt = -1, nxt_fl = 0, nxt_id = 0;
     if (cur >= 0) { nxt = it.next(dec); nxt_fl = it.flags; nxt_id = it.value; }
+    FA_TRACE_ONLY(if (gi == 0) FA_STAMP(g_trace_dkdv, 2, FA_CLOCK());)
     if (cur >= 0) {
       if (DOC) fetch_idx(cur);
       load_tile(cur, 0);
@@ -554,9 +563,11 @@ void bwd_dkdv_kernel(const KArgs a) {
       if (nxt >= 0) { nxt2 = it.next(dec); nxt2_fl = it.flags; nxt2_id = it.value; }
       wait_async_loads();
       __syncthreads();
+      FA_TRACE_ONLY(if (!tr_first) { FA_STAMP(g_trace_dkdv, 3, FA_CLOCK()); tr_first = true; })
       if (nxt >= 0) load_tile(nxt, 1);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
       compute(0, cur, cur_fl, cur_id);
+      FA_TRACE_ONLY(++tr_tiles;)
       cur = nxt; cur_fl = nxt_fl; cur_id = nxt_id; nxt = nxt2; nxt_fl = nxt2_fl; nxt_id = nxt2_id;
       if (cur < 0) break;
       nxt2 = -1;
@@ -566,10 +577,12 @@ void bwd_dkdv_kernel(const KArgs a) {
       if (nxt >= 0) load_tile(nxt, 0);
       if (DOC && nxt2 >= 0) fetch_idx(nxt2);
       compute(1, cur, cur_fl, cur_id);
+      FA_TRACE_ONLY(++tr_tiles;)
       cur = nxt; cur_fl = nxt_fl; cur_id = nxt_id; nxt = nxt2; nxt_fl = nxt2_fl; nxt_id = nxt2_id;
     }
   }
 
+  FA_STAMP(g_trace_dkdv, 4, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 6, tr_tiles);
   if (key < a.N) {
     T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs;
     T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
@@ -598,6 +611,7 @@ void bwd_dkdv_kernel(const KArgs a) {
       store(dkrow, acc2, a.scale);
     }
   }
+  FA_STAMP(g_trace_dkdv, 5, FA_CLOCK());
 }
 
 // Query tiles per workgroup (no ids) below which the 64-key role-split form is launched.
@@ -652,6 +666,10 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
     default: return -1;
   }
 }
+
+#ifdef FA_TRACE
+int trace_read_dkdv(long long* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace_dkdv), size_t(n) * 8); }
+#endif
 
 int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s) {
   return dtype == FA_DTYPE_BF16 ? launch_d<bf16_t>(a, D, causal, doc, s) : launch_d<fp16_t>(a, D, causal, doc, s);

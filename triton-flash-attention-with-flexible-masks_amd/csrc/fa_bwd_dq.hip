@@ -18,6 +18,11 @@ namespace fa {
 constexpr int kDqPre = 4;
 constexpr int kDqPre2 = 3;
 
+#ifdef FA_TRACE
+// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
+FA_TRACE_ARRAY(g_trace_dq);
+#endif
+
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 3 : 2, D <= 64 ? 3 : 2)))
 void bwd_dq_kernel(const KArgs a) {
@@ -32,6 +37,8 @@ void bwd_dq_kernel(const KArgs a) {
 
   const int lane = threadIdx.x & 63;
   const int g = lane >> 5;
+  FA_STAMP(g_trace_dq, 0, FA_CLOCK()); FA_STAMP(g_trace_dq, 4, 0); FA_STAMP(g_trace_dq, 7, -1);
+  FA_TRACE_ONLY(int tr_tiles = 0;)
 
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
   const int nSlots = nQt + (DOC ? split_extra(a) : 0);
@@ -48,6 +55,7 @@ void bwd_dq_kernel(const KArgs a) {
   int kt_first = qc.first_tile(a), kt_last = qc.last_tile(a);
   const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
+  FA_STAMP(g_trace_dq, 1, FA_CLOCK()); FA_STAMP(g_trace_dq, 7, (long long)wk.tile | ((long long)wk.split << 16) | ((long long)nsplit << 24));
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
 
@@ -204,6 +212,7 @@ void bwd_dq_kernel(const KArgs a) {
   };
   int cur = it.next(dec);
   int cur_fl = it.flags;
+  FA_STAMP(g_trace_dq, 2, FA_CLOCK());
   if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
     int nxt = it.next(dec);
@@ -211,6 +220,7 @@ void bwd_dq_kernel(const KArgs a) {
     __syncthreads();
     if (nxt >= 0) issue(1, nxt);
     compute(0, cur, cur_fl);
+    FA_TRACE_ONLY(++tr_tiles;)
     cur = nxt; cur_fl = it.flags;
     if (cur < 0) break;
     nxt = it.next(dec);
@@ -218,8 +228,10 @@ void bwd_dq_kernel(const KArgs a) {
     __syncthreads();
     if (nxt >= 0) issue(0, nxt);
     compute(1, cur, cur_fl);
+    FA_TRACE_ONLY(++tr_tiles;)
     cur = nxt; cur_fl = it.flags;
   }
+  FA_STAMP(g_trace_dq, 3, FA_CLOCK()); FA_STAMP(g_trace_dq, 5, tr_tiles);
 
   if (DOC && nsplit > 1) {
     // This workgroup saw one chunk of the keys: store the partial sum; the last chunk to arrive
@@ -235,7 +247,7 @@ void bwd_dq_kernel(const KArgs a) {
         f32x4 x = {dq[db][4 * q4 + 0], dq[db][4 * q4 + 1], dq[db][4 * q4 + 2], dq[db][4 * q4 + 3]};
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
-    if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
+    if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_dq, 4, FA_CLOCK()); return; }
     // (up to four chunks of four steps are requested together: every device-scope load is a round
     // trip of its own, so they are put in flight side by side instead of one after the other)
     constexpr int C4 = D / 4;
@@ -271,6 +283,7 @@ void bwd_dq_kernel(const KArgs a) {
           finish_row(mrow[u], (i0 + 256 * u) % C4, acc);
         }
       }
+      FA_STAMP(g_trace_dq, 4, FA_CLOCK());
       return;
     }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
@@ -284,6 +297,7 @@ void bwd_dq_kernel(const KArgs a) {
       }
       finish_row(mrow, c, acc);
     }
+    FA_STAMP(g_trace_dq, 4, FA_CLOCK());
     return;
   }
 
@@ -301,6 +315,7 @@ void bwd_dq_kernel(const KArgs a) {
         *reinterpret_cast<typename E::vec4*>(drow + 32 * db + 8 * q4 + 4 * g) = x;
       }
   }
+  FA_STAMP(g_trace_dq, 4, FA_CLOCK());
 }
 
 
@@ -332,6 +347,10 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
     default: return -1;
   }
 }
+
+#ifdef FA_TRACE
+int trace_read_dq(long long* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace_dq), size_t(n) * 8); }
+#endif
 
 int launch_bwd_dq(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s) {
   return dtype == FA_DTYPE_BF16 ? launch_d<bf16_t>(a, D, causal, doc, s) : launch_d<fp16_t>(a, D, causal, doc, s);

@@ -91,6 +91,22 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget 
 
 constexpr int kPairSpinDefault = 1 << 14;
 
+// Clock stamps per workgroup, for the measurement build only (compiled with -DFA_TRACE into a library of its
+// own, libflash_mi355_trace.so, read by `bench.py --wg-trace`).  A traced kernel keeps eight 64-bit words per
+// workgroup in a device array (wall clock, 100 MHz) that fa_trace_read copies out.  In the product build the
+// macros expand to nothing.
+#ifdef FA_TRACE
+constexpr int kTraceWgs = 65536;
+#define FA_TRACE_ARRAY(name) __device__ long long name[8 * fa::kTraceWgs]
+#define FA_STAMP(buf, i, v) do { if (threadIdx.x == 0 && blockIdx.x < fa::kTraceWgs) buf[blockIdx.x * 8 + (i)] = (long long)(v); } while (0)
+#define FA_CLOCK() wall_clock64()
+#define FA_TRACE_ONLY(...) __VA_ARGS__
+#else
+#define FA_STAMP(buf, i, v) do {} while (0)
+#define FA_CLOCK() 0
+#define FA_TRACE_ONLY(...)
+#endif
+
 // Key position of a row's diagonal as the kernels use it: at least -1 (the row sees nothing), and
 // small enough that position + window never overflows.
 constexpr int kPosMax = 0x3fffffff;
@@ -353,6 +369,11 @@ int launch_fwd(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStrea
 int launch_bwd_delta(const KArgs& a, int dtype, int D, hipStream_t s);
 int launch_bwd_dq(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
 int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+#ifdef FA_TRACE
+int trace_read_fwd(long long* host, int n);
+int trace_read_dq(long long* host, int n);
+int trace_read_dkdv(long long* host, int n);
+#endif
 // the same four for fp32 tensors (fa_f32.hip)
 int launch_fwd_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s);
 int launch_bwd_delta_f32(const KArgs& a, int D, hipStream_t s);

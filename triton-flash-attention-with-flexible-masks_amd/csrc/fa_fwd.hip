@@ -30,6 +30,11 @@ namespace fa {
 constexpr int kFwdPre = 4;
 constexpr int kFwdPre2 = 4;
 
+#ifdef FA_TRACE
+// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
+FA_TRACE_ARRAY(g_trace_fwd);
+#endif
+
 template <typename Tag, int D, bool CAUSAL, bool DOC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 3 : 2, D <= 64 ? 3 : 2)))
 void fwd_kernel(const KArgs a) {
@@ -44,6 +49,8 @@ void fwd_kernel(const KArgs a) {
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 5;
+  FA_STAMP(g_trace_fwd, 0, FA_CLOCK()); FA_STAMP(g_trace_fwd, 4, 0); FA_STAMP(g_trace_fwd, 7, -1);
+  FA_TRACE_ONLY(int tr_tiles = 0;)
 
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
   // order and see the longest key ranges; without ids the last rows do
@@ -62,6 +69,7 @@ void fwd_kernel(const KArgs a) {
   int kt_first = qc.first_tile(a), kt_last = qc.last_tile(a);
   const int nsplit = split_range(a, wk, kt_first, kt_last);
   if (wk.split >= nsplit) return;
+  FA_STAMP(g_trace_fwd, 1, FA_CLOCK()); FA_STAMP(g_trace_fwd, 7, (long long)wk.tile | ((long long)wk.split << 16) | ((long long)nsplit << 24));
   const int row = qc.row, rowc = qc.rowc, eq_i = qc.eq_i;
   const int* ekp = qc.ekp;
 
@@ -259,6 +267,7 @@ void fwd_kernel(const KArgs a) {
   };
   int cur = it.next(dec);
   int cur_fl = it.flags;
+  FA_STAMP(g_trace_fwd, 2, FA_CLOCK());
   if (cur >= 0) issue(0, cur);
   while (cur >= 0) {
     int nxt = it.next(dec);
@@ -266,6 +275,7 @@ void fwd_kernel(const KArgs a) {
     __syncthreads();
     if (nxt >= 0) issue(1, nxt);
     compute(0, cur, cur_fl);
+    FA_TRACE_ONLY(++tr_tiles;)
     cur = nxt; cur_fl = it.flags;
     if (cur < 0) break;
     nxt = it.next(dec);
@@ -273,8 +283,10 @@ void fwd_kernel(const KArgs a) {
     __syncthreads();
     if (nxt >= 0) issue(0, nxt);
     compute(1, cur, cur_fl);
+    FA_TRACE_ONLY(++tr_tiles;)
     cur = nxt; cur_fl = it.flags;
   }
+  FA_STAMP(g_trace_fwd, 3, FA_CLOCK()); FA_STAMP(g_trace_fwd, 5, tr_tiles);
 
   const float l_tot = xhalf_sum(l_run);
   if (DOC && nsplit > 1) {
@@ -293,7 +305,7 @@ void fwd_kernel(const KArgs a) {
         f32x4 x = {o[db][4 * q4 + 0], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]};
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
-    if (!split_arrive(a.sk_cnt + tbase, nsplit)) return;
+    if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_fwd, 4, FA_CLOCK()); return; }
     // merge: the whole workgroup walks the tile, one float4 of one row per thread and step.  The
     // partial results come through device-scope loads, each a round trip of its own: up to four chunks
     // of four steps are requested together (16 + 16 loads in flight per thread) instead of one by one.
@@ -343,6 +355,7 @@ void fwd_kernel(const KArgs a) {
           finish_row(mrow[u], (i0 + 256 * u) % C4, mmax, lsum, acc);
         }
       }
+      FA_STAMP(g_trace_fwd, 4, FA_CLOCK());
       return;
     }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
@@ -367,6 +380,7 @@ void fwd_kernel(const KArgs a) {
       }
       finish_row(mrow, c, mmax, lsum, acc);
     }
+    FA_STAMP(g_trace_fwd, 4, FA_CLOCK());
     return;
   }
 
@@ -386,6 +400,7 @@ void fwd_kernel(const KArgs a) {
         *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = x;
       }
   }
+  FA_STAMP(g_trace_fwd, 4, FA_CLOCK());
 }
 
 template <typename Tag, int D, bool CAUSAL, bool DOC>
@@ -416,6 +431,10 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
     default: return -1;
   }
 }
+
+#ifdef FA_TRACE
+int trace_read_fwd(long long* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace_fwd), size_t(n) * 8); }
+#endif
 
 int launch_fwd(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s) {
   return dtype == FA_DTYPE_BF16 ? launch_d<bf16_t>(a, D, causal, doc, s) : launch_d<fp16_t>(a, D, causal, doc, s);
