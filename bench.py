@@ -312,8 +312,18 @@ def main():
                 assert rc == 0, f"probe failed with hipError {rc}"
                 rates.append(round(tf_.value, 1))
             out[label] = rates
+        # the forward's phase structure without memory: ns per round, and the rate that is for a 128 x 64 x 128 tile per workgroup
+        probe.fa_probe_phase_time.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+        phase = {}
+        for label, wgs, soft in (("mfma_only_1wg", 1, 0), ("mfma_only_2wg", 2, 0), ("with_softmax_1wg", 1, 1), ("with_softmax_2wg", 2, 1)):
+            ns = ctypes.c_float(0)
+            rc = probe.fa_probe_phase_time(wgs, soft, 20000, ctypes.byref(ns))
+            assert rc == 0, f"probe failed with hipError {rc}"
+            phase[label] = {"ns_per_round": round(ns.value, 1),
+                            "tflops": round(256 * wgs * 4 * 32 * 32768.0 / ns.value * 1e-3, 1)}
         print(json.dumps({"probe": "v_mfma_f32_32x32x16_bf16, 8 workgroups of 4 waves per CU, 4 accumulators per wave",
-                          "tflops": out, "datasheet_peak": PEAK_TFLOPS["bf16"]}))
+                          "tflops": out, "datasheet_peak": PEAK_TFLOPS["bf16"],
+                          "forward_phase_structure_without_memory": phase}))
         return
     import torch
     from flash_mi355 import attention, workloads as W

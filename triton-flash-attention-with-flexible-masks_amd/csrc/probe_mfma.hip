@@ -68,3 +68,87 @@ extern "C" int fa_probe_mfma_rate(int random_operands, int iters, float* tflops)
   if (e == hipSuccess && ms > 0.f) *tflops = (float)((double)blocks * 4 * iters * 4 * 32768.0 / ms * 1e-9);
   return (int)e;
 }
+
+// The phase structure of the forward's tile loop without any memory access: per wave and round 16 MFMAs
+// in 2 chains (the scores), a vector phase that needs their results (32 x fma, exp2, add and 16
+// conversions: the softmax of a 64-key tile on its fast path), 16 MFMAs in 4 chains that need those
+// (P V), a workgroup barrier.  What this loop reaches is what the forward's instruction mix allows
+// before it reads a single operand.
+template <int SOFTMAX>
+__global__ __launch_bounds__(256) void phase_loop(float* out, int iters, int never) {
+  extern __shared__ char smem[];
+  if (never == 12345) smem[threadIdx.x] = 1;
+  bf16x8 q[8], kf, vf;
+  for (int j = 0; j < 8; ++j)
+    for (int i = 0; i < 8; ++i) q[j][i] = (__bf16)(0.01f * (threadIdx.x % 7 + i + j));
+  for (int i = 0; i < 8; ++i) { kf[i] = (__bf16)(0.02f * (threadIdx.x % 5 + i)); vf[i] = (__bf16)(0.03f * (threadIdx.x % 3 + i)); }
+  f32x16 o[4] = {{0}, {0}, {0}, {0}};
+  float m = 0.f, l = 0.f;
+  for (int it = 0; it < iters; ++it) {
+    f32x16 s0 = {0}, s1 = {0};
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[ks], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, q[ks], s1, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    bf16x8 p[4];
+    if (SOFTMAX) {
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float a = __builtin_amdgcn_exp2f(s0[i] * 0.125f - m), b = __builtin_amdgcn_exp2f(s1[i] * 0.125f - m);
+        sum += a + b;
+        p[i / 8][i % 8] = (__bf16)a;
+        p[2 + i / 8][i % 8] = (__bf16)b;
+      }
+      l += sum;
+      if (__builtin_expect(sum > 4096.f, 0)) m += 1.f;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { p[i / 8][i % 8] = (__bf16)s0[i]; p[2 + i / 8][i % 8] = (__bf16)s1[i]; }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db & 1 ? vf : kf, p[kk], o[db], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+  }
+  float s = l + m;
+  for (int d = 0; d < 4; ++d)
+    for (int i = 0; i < 16; ++i) s += o[d][i];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// One timed launch of `wgs_per_cu` (1 or 2) workgroups of 4 waves per CU, held to that residency by
+// their LDS size.  Returns 0 and the time of one round in ns (with 2 workgroups: of one round of
+// each), or the hipError_t that stopped it.
+extern "C" int fa_probe_phase_time(int wgs_per_cu, int softmax, int iters, float* ns_per_round) {
+  hipDeviceProp_t p;
+  hipError_t e = hipGetDeviceProperties(&p, 0);
+  if (e != hipSuccess) return (int)e;
+  if (wgs_per_cu != 1 && wgs_per_cu != 2) return (int)hipErrorInvalidValue;
+  const int lds = wgs_per_cu == 1 ? 150 * 1024 : 70 * 1024;
+  const int blocks = p.multiProcessorCount * wgs_per_cu;
+  auto kern = softmax ? phase_loop<1> : phase_loop<0>;
+  float* d = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  float ms = 0.f;
+  if ((e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds)) == hipSuccess &&
+      (e = hipMalloc(&d, size_t(blocks) * 256 * 4)) == hipSuccess && (e = hipEventCreate(&e0)) == hipSuccess &&
+      (e = hipEventCreate(&e1)) == hipSuccess) {
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, 0, d, 16, 0);   // warm
+    (void)hipEventRecord(e0, 0);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, 0, d, iters, 0);
+    (void)hipEventRecord(e1, 0);
+    if ((e = hipEventSynchronize(e1)) == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (d) (void)hipFree(d);
+  if (e == hipSuccess && ms > 0.f) *ns_per_round = ms * 1e6f / iters;
+  return (int)e;
+}
