@@ -367,6 +367,78 @@ def test_negative_and_large_scale():
     _run_case(1, 2, 1, 256, 2304, 64, torch.bfloat16, True, True, seed=54, sm_scale=0.3)   # split tiles + sharp softmax
 
 
+def _stress_inputs(kind, B, H, M, N, D, g):
+    """Inputs that push the online softmax: scores that grow or fall along the keys, outliers, a large
+    common offset, single dominating keys, tiny scores, one large score at the end of every key tile."""
+    q = torch.randn(B, H, M, D, generator=g)
+    k = torch.randn(B, H, N, D, generator=g)
+    if kind == "ramp_up":
+        q[..., 0] = 4.0
+        k[..., 0] = torch.linspace(-12, 12, N)[None, None]
+    elif kind == "ramp_down":
+        q[..., 0] = 4.0
+        k[..., 0] = torch.linspace(12, -12, N)[None, None]
+    elif kind == "outliers":
+        q = torch.where(torch.rand(q.shape, generator=g) < 0.01, q * 20, q)
+        k = torch.where(torch.rand(k.shape, generator=g) < 0.01, k * 20, k)
+    elif kind == "offset":
+        q, k = q + 3.0, k + 3.0
+    elif kind == "peaked":
+        k[:, :, ::97] *= 8.0
+    elif kind == "tiny":
+        q, k = q * 1e-3, k * 1e-3
+    elif kind == "saw":
+        q[..., 0] = 3.0
+        k[..., 0] = (torch.arange(N) % 64 == 63).float()[None, None] * 30.0
+    else:
+        raise KeyError(kind)
+    return q, k
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("kind", ["ramp_up", "ramp_down", "outliers", "offset", "peaked", "tiny", "saw"])
+def test_score_distributions_that_stress_the_online_softmax(kind, dtype):
+    """The reference point of the softmax moves lazily (only when a partial row sum leaves its bound), so
+    inputs that are not N(0,1) matter: no NaN, rows without keys agree, O and LSE inside the usual bounds.
+    The gradient bound of tests/_tol.py is stated for N(0,1) inputs; dQ = scale dS K and dK = scale dS^T Q
+    carry the error floor of dS (set by the 16-bit storage of O and P) times the size of K and Q, so here the
+    bound is scaled by the largest |q|, |k| element (dV: by 2, its P^T dO sums run over rows that all point at one key)."""
+    from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    from tests._tol import worst_ratio
+    for (B, H, M, N, D, causal, doc) in ((1, 2, 384, 384, 128, True, True), (1, 2, 300, 1100, 64, True, False),
+                                         (1, 1, 256, 2304, 128, False, True), (1, 2, 520, 520, 32, True, True)):
+        g = torch.Generator().manual_seed(7)
+        rng = np.random.default_rng(7)
+        q, k = (t.to(dtype) for t in _stress_inputs(kind, B, H, M, N, D, g))
+        v = torch.randn(B, H, N, D, generator=g).to(dtype)
+        do = torch.randn(B, H, M, D, generator=g).to(dtype)
+        eq = ek = None
+        mode = 0
+        if doc:
+            mode = SCORE_FUNC_MODE1_DOC
+            ek = torch.from_numpy(_ids(rng, B, H, N, "uniform"))[:, None, :].expand(B, H, N)
+            eq = ek[:, :, N - M:]
+        print(f"case {kind} {dtype} M{M} N{N} D{D} causal={causal} doc={doc}", flush=True)
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        eqd, ekd = (eq.cuda(), ek.cuda()) if doc else (None, None)
+        out, lse = attention_with_lse(qd.detach(), kd.detach(), vd.detach(), causal, None, eqd, ekd, mode)
+        attention(qd, kd, vd, causal, None, eqd, ekd, mode).backward(do.cuda())
+        torch.cuda.synchronize()
+        ref_o, ref_lse, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, causal, None, eq, ek, mode)
+        dead = torch.isinf(ref_lse)
+        assert torch.equal(torch.isinf(lse.cpu()), dead)
+        assert (out.float().cpu() - ref_o).abs().max().item() <= TOL_O
+        rel = (lse.cpu()[~dead] - ref_lse[~dead]).abs() / ref_lse[~dead].abs().clamp(min=1.0)
+        assert rel.max().item() <= TOL_LSE
+        size = max(1.0, q.float().abs().max().item(), k.float().abs().max().item())
+        for name, got, ref, factor in (("dq", qd.grad, ref_dq, size), ("dk", kd.grad, ref_dk, size), ("dv", vd.grad, ref_dv, 2.0)):
+            assert not torch.isnan(got).any(), name
+            r, err, at = worst_ratio(got, ref)
+            print(f"  {name}: worst err/bound {r:.3f} of {factor:.1f} allowed (err {err:.4g} at ref {at:.4g})", flush=True)
+            assert r <= factor, f"{name}: error {err:.5g} at reference value {at:.5g}"
+
+
 @pytest.mark.parametrize("dq_forms_delta", [False, True])
 def test_graph_capture_and_replay(dq_forms_delta):
     """The calls of a step (plan, forward, delta, dk/dv, dq -- or plan, forward, dq forming delta, dk/dv)
