@@ -903,17 +903,31 @@ def test_random_shapes_with_per_row_positions(seed):
               tol_o=TOL_F32 if f32 else TOL_O, tol_lse=TOL_F32 if f32 else TOL_LSE)
 
 
-@pytest.mark.xfail(strict=False, reason="one element of dK lands 3 % over the per-element bound: a finding, kept visible")
-def test_case_found_outside_the_bound():
-    """Found by a sweep of about 1500 random cases outside this suite (identical before and after the
-    per-row-position work, so not a regression): grouped heads, bf16, local ids, window 876, M 243 against
-    N 1419.  One element of dK comes out as -3.1875 where the exact value is -3.2081: 0.0128 of error from the
-    16-bit storage of P and dS inside the kernel plus the output's own rounding (a bf16 step is 0.0156 there),
-    0.0206 in all against the bound of 0.02.  The CPU model of the storage roundings
-    (oracle.attention_grads(store_dtype=...)) with the output rounding on top stays at 0.76 of the bound on the
-    same inputs, so the kernel is somewhat worse than that model here.  Every other element of the case, and
-    every case of the suite, is inside the bound."""
+def test_p_crosses_the_wave_pair_as_fp16():
+    """In the role-split dk/dv form (D = 128) the gradient wave forms dS = P (dP - delta) from the P that the
+    score wave hands over through LDS.  While that copy was in the element type, bf16 tensors carried one
+    rounding more than the reference (which multiplies its fp32 P, flash_triton.py:301), and a sweep of random
+    cases found dK elements up to 19 % over the per-element bound (this case: 0.0206 against 0.02 at an exact
+    value of -3.2081; grouped heads, local ids, window 876).  P <= 1 crosses as fp16 now, for either element
+    type: 11 significant bits in the same two bytes.  The case sits at 0.65 of the bound."""
     _run_case(1, 4, 2, 243, 1419, 128, torch.bfloat16, True, True, seed=5012, ids_kind="alllocal", window=876)
+    _run_case(2, 2, 1, 651, 617, 128, torch.bfloat16, False, True, seed=5086, ids_kind="alllocal")
+    _run_case(2, 4, 2, 248, 1297, 128, torch.bfloat16, True, True, seed=5210, ids_kind="alllocal", prefix=530)
+
+
+@pytest.mark.xfail(strict=False, reason="one element of dK lands 17 % over the per-element bound, at the error floor "
+                                        "that the 16-bit storage of O sets through delta: a finding, kept visible")
+def test_case_found_outside_the_bound():
+    """Found by a sweep of about 3000 random cases outside this suite: grouped heads, bf16, documents of 8-96
+    tokens, window 96, M 563 against N 879.  One element of dK comes out as 0.9727 where the exact value is
+    0.9492 (0.0235 against the bound of 0.02).  With rows that see a few dozen keys P is large, and the error
+    that the 16-bit storage of O puts into delta = rowsum(O dO) reaches dS = P (dP - delta) undamped; the
+    reference forms delta from the stored O as well (flash_triton.py:165).  The CPU model of the reference's
+    storage roundings (oracle.attention_grads(store_dtype=...), output rounded too) reaches 0.92 of the bound
+    on the same inputs, at another element; the kernel's O differs from the model's by one bf16 step in places
+    (other summation order), which makes its delta another draw from the same error distribution.  Every
+    other element of the case, and every case of the suite, is inside the bound; the bound is not widened."""
+    _run_case(2, 4, 2, 563, 879, 128, torch.bfloat16, True, True, seed=5128, ids_kind="alllocal", window=96)
 
 
 @pytest.mark.parametrize("seed", list(range(200, 232)))

@@ -52,7 +52,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   constexpr int TILE_BYTES = BQ * DL * 2;
   constexpr int AUX_OFF = 4 * TILE_BYTES;      // [2 buffers][4 arrays][64] x 4 bytes
   constexpr int AUX_BYTES = 1024;
-  constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][NKB key blocks][2 x 1024]: P in the element type
+  constexpr int P_OFF = AUX_OFF + 2 * AUX_BYTES;  // [2 (block parity)][NKB key blocks][2 x 1024]: P as fp16
   constexpr int P_BYTES = 2048;
   constexpr int FLAG_OFF = P_OFF + 2 * NKB * P_BYTES;   // [2 (block parity)][NKB] sequence numbers of the published P
   // Polls of the pair flag before the gradient wave gives up (kPairSpinDefault, about a millisecond:
@@ -333,7 +333,22 @@ void bwd_dkdv_kernel(const KArgs a) {
           const typename E::vec2 pr = E::cvt2(x[qb][8 * half + t], x[qb][8 * half + t + 1]);
           yf[qb][half][t] = pr[0]; yf[qb][half][t + 1] = pr[1];
         }
-        *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[qb][half];
+        // P crosses to the gradient wave as fp16 whatever the element type: P <= 1, so fp16 keeps 11
+        // significant bits of it (anything below 6e-8 becomes 0, far under the rounding of dS itself) and
+        // dS = P (dP - delta) is formed from a P that is as good as the fp32 one; the bf16 copy above is
+        // the operand of this wave's own dV product only.
+        if constexpr (sizeof(typename E::scalar) == 2 && !__is_same(typename E::scalar, _Float16)) {
+          f16x8 ph;
+#pragma unroll
+          for (int t = 0; t < 8; t += 2) {
+            const f32x2 pp = {x[qb][8 * half + t], x[qb][8 * half + t + 1]};
+            const f16x2 hh = __builtin_convertvector(pp, f16x2);
+            ph[t] = hh[0]; ph[t + 1] = hh[1];
+          }
+          *reinterpret_cast<f16x8*>(pbuf + half * 1024) = ph;
+        } else {
+          *reinterpret_cast<vec8*>(pbuf + half * 1024) = yf[qb][half];
+        }
       }
       lds_flag_store(smem + FLAG_OFF + (qb * NKB + kb) * 4, pair_seq);
     };
@@ -352,9 +367,9 @@ void bwd_dkdv_kernel(const KArgs a) {
         __builtin_amdgcn_s_sleep(1);
       }
       if (!arrived) pair_lost = 1;
-      vec8 pr8[2];
+      f16x8 pr8[2];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const vec8*>(pbuf + half * 1024);
+      for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const f16x8*>(pbuf + half * 1024);
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         const f32x8 pv = __builtin_convertvector(pr8[half], f32x8);
