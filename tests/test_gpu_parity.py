@@ -915,19 +915,39 @@ def test_p_crosses_the_wave_pair_as_fp16():
     _run_case(2, 4, 2, 248, 1297, 128, torch.bfloat16, True, True, seed=5210, ids_kind="alllocal", prefix=530)
 
 
-@pytest.mark.xfail(strict=False, reason="one element of dK lands 17 % over the per-element bound, at the error floor "
-                                        "that the 16-bit storage of O sets through delta: a finding, kept visible")
-def test_case_found_outside_the_bound():
-    """Found by a sweep of about 3000 random cases outside this suite: grouped heads, bf16, documents of 8-96
-    tokens, window 96, M 563 against N 879.  One element of dK comes out as 0.9727 where the exact value is
-    0.9492 (0.0235 against the bound of 0.02).  With rows that see a few dozen keys P is large, and the error
-    that the 16-bit storage of O puts into delta = rowsum(O dO) reaches dS = P (dP - delta) undamped; the
-    reference forms delta from the stored O as well (flash_triton.py:165).  The CPU model of the reference's
-    storage roundings (oracle.attention_grads(store_dtype=...), output rounded too) reaches 0.92 of the bound
-    on the same inputs, at another element; the kernel's O differs from the model's by one bf16 step in places
-    (other summation order), which makes its delta another draw from the same error distribution.  Every
-    other element of the case, and every case of the suite, is inside the bound; the bound is not widened."""
-    _run_case(2, 4, 2, 563, 879, 128, torch.bfloat16, True, True, seed=5128, ids_kind="alllocal", window=96)
+FLOOR_CASES = [
+    # B, H, Hk, M, N, D, seed, window, per-head ids, positions
+    (2, 4, 2, 563, 879, 128, 5128, 96, False, None),
+    (2, 2, 1, 180, 5, 64, 1429, 0, True, "steps"),
+    (2, 2, 2, 215, 4, 128, 1433, 64, False, "steps"),
+    (1, 2, 1, 499, 4, 64, 1307, 64, False, "steps"),
+]
+
+
+@pytest.mark.xfail(strict=False, reason="dK elements over the per-element bound (by 9-17 %, one case by 92 %), at the error floor "
+                                        "that the 16-bit storage of O, P and dS sets: a finding, kept visible")
+@pytest.mark.parametrize("case", FLOOR_CASES, ids=lambda c: "M%d-N%d-D%d-seed%d" % (c[3], c[4], c[5], c[6]))
+def test_case_found_outside_the_bound(case):
+    """Found by sweeps of about 3500 random cases outside this suite (bf16, local ids).  What they share: rows
+    that keep very few keys, so P is close to 1, and dK elements that sum over many such rows.
+    First case (documents of 8-96 tokens, window 96): one element of dK comes out as 0.9727 where the exact
+    value is 0.9492 (0.0235 against the bound of 0.02).  The error that the 16-bit storage of O puts into
+    delta = rowsum(O dO) reaches dS = P (dP - delta) undamped when P is large; the reference forms delta from
+    the stored O as well (flash_triton.py:165).  The CPU model of the reference's storage roundings
+    (oracle.attention_grads(store_dtype=...), output rounded too) reaches 0.92 of the bound on the same inputs
+    at another element; the kernel's O differs from the model's by one bf16 step in places (other summation
+    order), which makes its delta another draw from the same error distribution.
+    Second and third case (5 and 4 keys in all, 180 and 215 query rows with per-row positions, 1.0-1.6 kept keys
+    per row, 55 rows per key): 1.09 of the bound -- and the CPU model of the reference's roundings is itself at
+    1.06 and 1.09 of it there: no implementation that rounds where the reference rounds meets the bound on
+    these inputs.  Fourth case (4 keys, 499 rows, two query heads per key head, every id global: 4 kept keys per
+    row, a thousand terms per dK element): 1.92 of the bound, where the model of the reference's roundings is
+    at 2.40 for dK and 2.52 for dV (the reference rounds each head's dK, dV before the group sum,
+    flash_triton.py:635-637; the kernel sums the group in fp32).  Every other element of these cases, and every case of the suite, is inside the bound; the
+    bound is not widened."""
+    B, H, Hk, M, N, D, seed, window, per_head, qpos = case
+    _run_case(B, H, Hk, M, N, D, torch.bfloat16, True, True, seed=seed, ids_kind="allglobal" if seed == 1307 else "alllocal",
+              window=window, per_head_ids=per_head, qpos=qpos)
 
 
 @pytest.mark.parametrize("seed", list(range(200, 232)))
