@@ -358,6 +358,31 @@ def test_random_shapes(seed):
     _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed=seed, ids_kind=kind, per_head_ids=per_head, id_dtype=idt)
 
 
+def test_empty_inputs():
+    """No query rows, no batch, or no keys at all: nothing is launched; O has q's shape (zeros where there are
+    rows: a row without keys behaves as a row whose keys are all masked, O = 0 and LSE = -inf) and the
+    gradients are zeros of the operands' shapes.  (The reference cannot run these: its launcher refuses the
+    empty grid and its kernel divides 0 by 0 without keys.)"""
+    from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
+    dev = torch.device("cuda")
+    for (B, H, Hk, M, N, causal, doc) in ((1, 2, 2, 0, 64, False, False), (0, 2, 1, 32, 32, True, True),
+                                          (2, 4, 2, 48, 0, False, True), (1, 2, 2, 0, 0, True, False)):
+        q = torch.randn(B, H, M, 64, device=dev).bfloat16().requires_grad_(True)
+        k = torch.randn(B, Hk, N, 64, device=dev).bfloat16().requires_grad_(True)
+        v = torch.randn(B, Hk, N, 64, device=dev).bfloat16().requires_grad_(True)
+        eq = torch.zeros(B, H, M, dtype=torch.int32, device=dev) - 1 if doc else None
+        ek = torch.zeros(B, H, N, dtype=torch.int32, device=dev) - 1 if doc else None
+        out, lse = attention_with_lse(q, k, v, causal, None, eq, ek, SCORE_FUNC_MODE1_DOC if doc else 0)
+        assert out.shape == q.shape and out.dtype == q.dtype and lse.shape == (B, H, M)
+        assert out.abs().sum().item() == 0 and bool(torch.isinf(lse).all())
+        (out.float().sum() + 0 * lse.nan_to_num(neginf=0.0).sum()).backward()
+        for t in (q, k, v):
+            assert t.grad is not None and t.grad.shape == t.shape and t.grad.abs().sum().item() == 0
+        q.grad = None
+        attention(q, k, v, causal, None, eq, ek, SCORE_FUNC_MODE1_DOC if doc else 0).sum().backward()
+        assert q.grad.shape == q.shape
+
+
 def test_negative_and_large_scale():
     """sm_scale < 0 (the sign moves into Q so that the running maximum stays a maximum) and a large
     scale (sharp softmax: the lazily moved reference point has to move often)."""

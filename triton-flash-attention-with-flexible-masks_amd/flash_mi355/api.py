@@ -191,6 +191,14 @@ class _Impl:
                 "qpos must be an integer tensor [bs|1, Lq]"
             _check_same_device(q, qpos=qpos)
             qpos = qpos.to(torch.int32).contiguous()
+        ctx.nothing_to_do = B == 0 or H == 0 or M == 0 or N == 0
+        if ctx.nothing_to_do:
+            # No rows, or rows without a single key: nothing is launched (the C ABI refuses sizes <= 0).  A row
+            # without keys gives O = 0, LSE = -inf and no gradient, as a row whose keys are all masked does.
+            # (The reference launches an empty grid for Lq = 0, which its launcher refuses, and divides 0 by 0 for Lk = 0.)
+            ctx.like = (q.new_empty(0), k.shape, v.shape)
+            ctx.qshape = q.shape
+            return torch.zeros_like(q), torch.full((B, H, M), -math.inf, device=q.device, dtype=torch.float32)
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
 
         L = _cabi.lib()
@@ -212,6 +220,10 @@ class _Impl:
 
     @staticmethod
     def backward(ctx, do, dlse):
+        if ctx.nothing_to_do:
+            like, kshape, vshape = ctx.like
+            dq = like.new_zeros(ctx.qshape)
+            return dq, like.new_zeros(kshape), like.new_zeros(vshape), None, None, None, None, None, None, None, None
         q, k, v, o, lse, eq, ek, workspace, qpos = ctx.saved_tensors
         B, H, M, D, N, Hk, num_groups, MN_GAP = ctx.shapes
         score_func_mode, window, prefix = ctx.score_func_info
