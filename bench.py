@@ -216,9 +216,19 @@ def wg_trace(w, q, k, v, do, eq, ek, torch):
             "mean_loop_us": round(float(((live[:, c_loop] - live[:, c_setup]) * TICK_US).mean()), 2),
             "mean_drain_us": round(float(((live[:, c_end] - live[:, c_loop]) * TICK_US).mean()), 2),
             "mean_tiles": round(float(live[:, c_tiles].mean()), 2),
+            "max_tiles": int(live[:, c_tiles].max()),
+            "max_lifetime_us": round(float(life.max()), 1),
+            "last_start_us": round(float((t[:, c_start].max() - t[:, 0].min()) * TICK_US), 1),
             "loop_us_per_tile": round(float((live[:, c_loop] - live[:, c_setup]).sum() * TICK_US / live[:, c_tiles].sum()), 3),
             "mean_resident_per_cu": round(float(life.sum() / (span * 256)), 3),
         }
+        if which < 2:   # the workgroups that merged the chunks of a split tile: their drain in two parts
+            mg = live[live[:, 6] != 0]
+            if len(mg):
+                r["merging_workgroups"] = int(len(mg))
+                r["mean_store_and_arrive_us"] = round(float(((mg[:, 6] - mg[:, c_loop]) * TICK_US).mean()), 2)
+                r["mean_merge_us"] = round(float(((mg[:, c_end] - mg[:, 6]) * TICK_US).mean()), 2)
+                r["mean_chunks_merged"] = round(float(((mg[:, 7] >> 24) & 0xff).mean()), 2)
         if len(idle):
             r["mean_lifetime_no_tiles_us"] = round(float(((idle[:, c_end] - idle[:, c_start]) * TICK_US).mean()), 2)
         out[name] = r

@@ -257,6 +257,9 @@ def test_long_key_ranges_of_global_rows():
     _run_case(1, 2, 1, 300, 5000, 128, torch.float16, False, True, seed=22)
     _run_case(1, 1, 1, 1200, 2304, 128, torch.bfloat16, True, True, seed=23, ids_kind="allglobal")
     _run_case(2, 2, 2, 2048, 2048, 16, torch.bfloat16, True, True, seed=24)
+    # few query tiles in the launch: up to 16 chunks.  6 chunks (merged eight at a time) and 12 (merged one by one)
+    _run_case(1, 2, 2, 150, 6500, 128, torch.bfloat16, True, True, seed=25, ids_kind="allglobal")
+    _run_case(1, 2, 1, 64, 13000, 64, torch.float16, False, True, seed=26)
 
 
 def test_short_query_long_key_without_ids():

@@ -19,7 +19,7 @@ constexpr int kDqPre = 4;
 constexpr int kDqPre2 = 3;
 
 #ifdef FA_TRACE
-// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
+// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 6 (merging workgroup only) partial result stored and arrival counted, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
 FA_TRACE_ARRAY(g_trace_dq);
 #endif
 
@@ -37,7 +37,7 @@ void bwd_dq_kernel(const KArgs a) {
 
   const int lane = threadIdx.x & 63;
   const int g = lane >> 5;
-  FA_STAMP(g_trace_dq, 0, FA_CLOCK()); FA_STAMP(g_trace_dq, 4, 0); FA_STAMP(g_trace_dq, 7, -1);
+  FA_STAMP(g_trace_dq, 0, FA_CLOCK()); FA_STAMP(g_trace_dq, 4, 0); FA_STAMP(g_trace_dq, 6, 0); FA_STAMP(g_trace_dq, 7, -1);
   FA_TRACE_ONLY(int tr_tiles = 0;)
 
   const int nQt = DOC ? a.Pp / BM : (a.M + BM - 1) / BM;
@@ -248,8 +248,9 @@ void bwd_dq_kernel(const KArgs a) {
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_dq, 4, FA_CLOCK()); return; }
-    // (up to four chunks of four steps are requested together: every device-scope load is a round
-    // trip of its own, so they are put in flight side by side instead of one after the other)
+    FA_STAMP(g_trace_dq, 6, FA_CLOCK());
+    // (up to eight chunks are requested together, four or two steps of them: every device-scope load is a
+    // round trip of its own, so they are put in flight side by side instead of one after the other)
     constexpr int C4 = D / 4;
     const float* bo = a.sk_o + tbase * a.split_k * (128 * D);
     const int* prm = a.perm + b * a.pm_bs + h * a.pm_hs + wk.tile * 128;
@@ -259,8 +260,9 @@ void bwd_dq_kernel(const KArgs a) {
       typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
       *reinterpret_cast<typename E::vec4*>(dqp + int64_t(mrow) * a.dq_rs + 4 * c) = x;
     };
-    if (nsplit <= 4) {
-      constexpr int IT = 4, NS = 4;
+    // NS chunk slots of IT steps each: 16 loads in flight per thread whatever the number of chunks
+    auto merge_batched = [&](auto it_c, auto ns_c) __attribute__((always_inline)) {
+      constexpr int IT = decltype(it_c)::value, NS = decltype(ns_c)::value;
       for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
         f32x4 x[IT][NS];
         int mrow[IT];
@@ -283,6 +285,10 @@ void bwd_dq_kernel(const KArgs a) {
           finish_row(mrow[u], (i0 + 256 * u) % C4, acc);
         }
       }
+    };
+    if (nsplit <= 8) {   // (with 9 .. 16 chunks the plain loop below measured the same or better)
+      if (nsplit <= 4) merge_batched(IntC<4>{}, IntC<4>{});
+      else merge_batched(IntC<2>{}, IntC<8>{});
       FA_STAMP(g_trace_dq, 4, FA_CLOCK());
       return;
     }

@@ -51,6 +51,7 @@ constexpr int kPermAlign = 256;
 constexpr int kSplitMinTiles = 16;   // key tiles (of 64) per chunk below which splitting does not pay
 constexpr int kSplitKMax = 4;        // more chunks did not pay on any shape with enough query tiles to fill the chip
 constexpr int kSplitKMaxFew = 16;    // ... but they do when the whole launch is short of workgroups (few query rows)
+constexpr int kSplitFewWgs = 1024;   // query tiles in the launch (all heads) below which it counts as short of workgroups
 struct SplitCfg {
   int k;      // chunks per tile (1: nothing is ever split)
   int tiles;  // global-row tiles per (batch, head) that can be split
@@ -60,8 +61,8 @@ struct SplitCfg {
 // of them long.  The budget is a hard bound on the scratch part of the workspace: with many (batch,
 // head) pairs it buys fewer tiles per pair, down to none (such launches have workgroups to spare and
 // short key ranges per tile; with fewer than two tiles in the budget at 4 chunks, 2 chunks are tried).
-// With so few query rows that even kSplitKMax chunks per tile leave the chip short of workgroups
-// (decoding, the tail of a long prompt) the chunks go down to kSplitMinTiles key tiles, up to
+// With fewer than kSplitFewWgs query tiles in the whole launch (decoding, the tail of a long prompt, a short
+// query block against a long packed key sequence) the chunks go down to kSplitMinTiles key tiles, up to
 // kSplitKMaxFew of them.  Never more splittable tiles than M rows can fill.
 constexpr uint64_t kSplitScratchBudget = uint64_t(128) << 20;   // bytes of sk_ml + sk_o
 inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget = kSplitScratchBudget) {
@@ -70,8 +71,13 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget 
   if (nKs < 2 * kSplitMinTiles) return c;   // no key range can be long enough to be cut
   const int qtiles = (M + 127) / 128 + 1;   // 128-row tiles of global rows a (batch, head) can have
   const uint64_t wgs = uint64_t(B) * H * qtiles;
-  if (wgs * kSplitKMax < 512) {
-    const int kmax = int(512 / wgs) < kSplitKMaxFew ? (int(512 / wgs) > kSplitKMax ? int(512 / wgs) : kSplitKMax) : kSplitKMaxFew;
+  if (wgs < kSplitFewWgs) {
+    // Short of workgroups: the chunks of the global-row tiles are what fills the chip.  About 256 workgroups
+    // that each stream their own K / V chunk keep the memory system busy (more of them only add merge work),
+    // and every (batch, head) has at least one such tile.
+    const uint64_t bh = uint64_t(B) * H;
+    const int fill = int(256 / bh);
+    const int kmax = fill < kSplitKMax ? kSplitKMax : (fill > kSplitKMaxFew ? kSplitKMaxFew : fill);
     const int want = nKs / kSplitMinTiles;
     c.k = want < 2 ? 2 : (want > kmax ? kmax : want);
   } else {
@@ -88,6 +94,9 @@ inline SplitCfg split_config(int B, int H, int M, int N, int D, uint64_t budget 
   if (c.tiles <= 0) { c.tiles = 0; c.k = 1; }
   return c;
 }
+
+// Compile-time integer handed to a generic lambda.
+template <int V> struct IntC { static constexpr int value = V; };
 
 constexpr int kPairSpinDefault = 1 << 14;
 

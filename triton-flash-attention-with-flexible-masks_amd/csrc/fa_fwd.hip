@@ -31,7 +31,7 @@ constexpr int kFwdPre = 4;
 constexpr int kFwdPre2 = 4;
 
 #ifdef FA_TRACE
-// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
+// words: 0 start, 1 rows and ids known, 2 before the tile loop, 3 after it, 4 end, 5 key tiles computed, 6 (merging workgroup only) partial result stored and arrival counted, 7 tile | chunk << 16 | chunks << 24 (-1: left at once)
 FA_TRACE_ARRAY(g_trace_fwd);
 #endif
 
@@ -49,7 +49,7 @@ void fwd_kernel(const KArgs a) {
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 5;
-  FA_STAMP(g_trace_fwd, 0, FA_CLOCK()); FA_STAMP(g_trace_fwd, 4, 0); FA_STAMP(g_trace_fwd, 7, -1);
+  FA_STAMP(g_trace_fwd, 0, FA_CLOCK()); FA_STAMP(g_trace_fwd, 4, 0); FA_STAMP(g_trace_fwd, 6, 0); FA_STAMP(g_trace_fwd, 7, -1);
   FA_TRACE_ONLY(int tr_tiles = 0;)
 
   // heaviest tiles first: with ids the global-row tiles sit at the end of the permuted
@@ -306,9 +306,10 @@ void fwd_kernel(const KArgs a) {
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_fwd, 4, FA_CLOCK()); return; }
+    FA_STAMP(g_trace_fwd, 6, FA_CLOCK());
     // merge: the whole workgroup walks the tile, one float4 of one row per thread and step.  The
-    // partial results come through device-scope loads, each a round trip of its own: up to four chunks
-    // of four steps are requested together (16 + 16 loads in flight per thread) instead of one by one.
+    // partial results come through device-scope loads, each a round trip of its own: up to eight chunks are
+    // requested together, four or two steps of them (16 + 16 loads in flight per thread), instead of one by one.
     constexpr int C4 = D / 4;
     const float* bo = a.sk_o + tbase * a.split_k * (128 * D);
     const float* bml = a.sk_ml + tbase * a.split_k * (128 * 2);
@@ -321,8 +322,9 @@ void fwd_kernel(const KArgs a) {
       typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
       *reinterpret_cast<typename E::vec4*>(op + int64_t(mrow) * a.o_rs + 4 * c) = x;
     };
-    if (nsplit <= 4) {
-      constexpr int IT = 4, NS = 4;
+    // NS chunk slots of IT steps each: 16 + 16 loads in flight per thread whatever the number of chunks
+    auto merge_batched = [&](auto it_c, auto ns_c) __attribute__((always_inline)) {
+      constexpr int IT = decltype(it_c)::value, NS = decltype(ns_c)::value;
       for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
         float m_[IT][NS], l_[IT][NS];
         f32x4 x[IT][NS];
@@ -355,6 +357,10 @@ void fwd_kernel(const KArgs a) {
           finish_row(mrow[u], (i0 + 256 * u) % C4, mmax, lsum, acc);
         }
       }
+    };
+    if (nsplit <= 8) {   // (with 9 .. 16 chunks the plain loop below measured the same or better)
+      if (nsplit <= 4) merge_batched(IntC<4>{}, IntC<4>{});
+      else merge_batched(IntC<2>{}, IntC<8>{});
       FA_STAMP(g_trace_fwd, 4, FA_CLOCK());
       return;
     }
