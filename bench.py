@@ -229,6 +229,9 @@ def wg_trace(w, q, k, v, do, eq, ek, torch):
                 r["mean_store_and_arrive_us"] = round(float(((mg[:, 6] - mg[:, c_loop]) * TICK_US).mean()), 2)
                 r["mean_merge_us"] = round(float(((mg[:, c_end] - mg[:, 6]) * TICK_US).mean()), 2)
                 r["mean_chunks_merged"] = round(float(((mg[:, 7] >> 24) & 0xff).mean()), 2)
+        if which == 2 and live[:, 1].any():   # role-split dk/dv: what its first gradient wave waits for the score wave's P
+            r["mean_pair_wait_shader_clocks"] = round(float(live[:, 1].mean()), 0)
+            r["mean_pair_wait_clocks_per_tile"] = round(float(live[:, 1].sum() / live[:, c_tiles].sum()), 1)
         if len(idle):
             r["mean_lifetime_no_tiles_us"] = round(float(((idle[:, c_end] - idle[:, c_start]) * TICK_US).mean()), 2)
         out[name] = r

@@ -36,7 +36,7 @@ constexpr int kKvPre2 = 3;
 //                never leaves the registers and the only barrier is the one of the tile stream; two
 //                workgroups share a CU.
 #ifdef FA_TRACE
-// words: 0 start, 1 K / V fragments requested, 2 first query tile chosen, 3 first query tile in LDS, 4 after the tile loop, 5 end, 6 query tiles computed, 7 key tile | (batch, kv head) << 16 (-1: left at once)
+// words: 0 start, 1 shader clocks the first gradient wave waited for P (role-split form), 2 first query tile chosen, 3 first query tile in LDS, 4 after the tile loop, 5 end, 6 query tiles computed, 7 key tile | (batch, kv head) << 16 (-1: left at once)
 FA_TRACE_ARRAY(g_trace_dkdv);
 #endif
 
@@ -69,7 +69,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   const int role = SPLIT ? wave / NKB : 0, kb = wave % NKB;
   const int lq = lane & 31, g = lane >> 5;
   FA_STAMP(g_trace_dkdv, 0, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 5, 0); FA_STAMP(g_trace_dkdv, 7, -1);
-  FA_TRACE_ONLY(int tr_tiles = 0; bool tr_first = false;)
+  FA_TRACE_ONLY(int tr_tiles = 0; bool tr_first = false; long long tr_wait = 0;)
 
   // one workgroup per (key tile, batch, kv head)
   const int nKt = (a.N + BK - 1) / BK;
@@ -101,7 +101,7 @@ void bwd_dkdv_kernel(const KArgs a) {
   // 128-key form, which serves long streams, that gave the faster loop (4.24 against 4.39 ms, plain
   // causal 16K); at D <= 64 the difference stayed inside the run-to-run spread.
   constexpr bool LATE_SETTLE = SPLIT && NKB == 2;
-  FA_STAMP(g_trace_dkdv, 1, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 7, (long long)kt | ((long long)bhk << 16));
+  FA_STAMP(g_trace_dkdv, 1, 0); FA_STAMP(g_trace_dkdv, 7, (long long)kt | ((long long)bhk << 16));
   if (!LATE_SETTLE) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { settle(frag[ks]); if (!SPLIT) settle(frag2[ks]); }
@@ -362,11 +362,13 @@ void bwd_dkdv_kernel(const KArgs a) {
       for (int q4 = 0; q4 < 4; ++q4) dl[q4] = *reinterpret_cast<const f32x4*>(aux + 256 + (32 * qb + 8 * q4 + 4 * g) * 4);
       const char* fl = smem + FLAG_OFF + (qb * NKB + kb) * 4;
       bool arrived = false;
+      FA_TRACE_ONLY(const long long tr_t0 = __builtin_readcyclecounter();)
       for (int spin = 0; spin <= pair_spin_max; ++spin) {
         if (__builtin_amdgcn_readfirstlane(lds_flag_load(fl)) == pair_seq) { arrived = true; break; }
         __builtin_amdgcn_s_sleep(1);
       }
       if (!arrived) pair_lost = 1;
+      FA_TRACE_ONLY(tr_wait += __builtin_readcyclecounter() - tr_t0;)
       f16x8 pr8[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) pr8[half] = *reinterpret_cast<const f16x8*>(pbuf + half * 1024);
@@ -598,6 +600,8 @@ void bwd_dkdv_kernel(const KArgs a) {
   }
 
   FA_STAMP(g_trace_dkdv, 4, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 6, tr_tiles);
+  // shader clocks the first gradient wave spent at the pair flag (role-split form)
+  FA_TRACE_ONLY(if (SPLIT && threadIdx.x == 64 * NKB && blockIdx.x < fa::kTraceWgs) g_trace_dkdv[blockIdx.x * 8 + 1] = tr_wait;)
   if (key < a.N) {
     T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs;
     T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
