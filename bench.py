@@ -23,6 +23,8 @@ the matrix pipes can do, never above 1.  The mask plan lets the kernels skip mos
 canonical tiles, so the tile-effective rate of the same launch (what ``value``
 counts) is higher and is reported beside it.  ``pct_of_mfma_peak`` is the executed
 rate of the whole step; ``pct_of_mfma_peak_tile_effective`` the north-star figure.
+``roofline.sustained_mfma_probe`` is what a bare MFMA loop on random bf16 operands sustains on the same box
+right after the timed region (``frac_of_sustained`` = achieved over that): context only, ``frac`` is what counts.
 ``cpu_baseline`` times the reference's eager mask-materialising path on the host
 cores for a bounded sample (a few heads) of the same workload.
 """
@@ -413,6 +415,20 @@ def main():
                             "frac": round(tf(executed[n], kt[n]) / peak, 4),
                             "avg_launch_ms": round(kt[n], 4),
                             "tile_effective_tflops": round(tf(u * f_fwd["tile"], kt[n]), 1)} for n, u in gemm_units.items()}}
+
+    if w.dtype in ("bf16", "fp16"):
+        # What the matrix pipes of THIS box sustain in a bare MFMA loop on random operands (the boxes of a pool
+        # differ, and the clock follows the load): context for `frac`, which stays a share of the data-sheet peak.
+        try:
+            from flash_mi355.build import PROBE_LIB_PATH
+            probe = ctypes.CDLL(str(PROBE_LIB_PATH))
+            probe.fa_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+            rate = ctypes.c_float(0)
+            if probe.fa_probe_mfma_rate(1, 20000, ctypes.byref(rate)) == 0 and rate.value > 0:
+                roofline["sustained_mfma_probe"] = round(rate.value, 1)
+                roofline["frac_of_sustained"] = round(roofline["achieved"] / rate.value, 4)
+        except OSError:
+            pass
 
     value = tf(3.5 * f_fwd["tile"], ms_per_step)
     executed_step = ex["fwd"] + ex["dq"] + ex["dkdv"]
