@@ -361,6 +361,46 @@ def test_random_shapes(seed):
     _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed=seed, ids_kind=kind, per_head_ids=per_head, id_dtype=idt)
 
 
+def test_clock_stamp_build_gives_the_same_bits():
+    """The measurement build (the same sources with -DFA_TRACE, what `bench.py --wg-trace` loads) must time the
+    kernels the product runs: its forward, dq and dk/dv results equal the product library's bit for bit."""
+    import ctypes
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    from flash_mi355.build import TRACE_LIB_PATH
+    T = ctypes.CDLL(str(TRACE_LIB_PATH))
+    L = _cabi.lib()
+    B, H, M, D = 1, 2, 2304, 128
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(91)
+    rng = np.random.default_rng(91)
+    ids = torch.from_numpy(_ids(rng, B, H, M, "uniform")).to(dev)[:, None, :].expand(B, H, M)
+    q, k, v, do = (torch.randn(B, H, M, D, generator=g).bfloat16().to(dev) for _ in range(4))
+    results = []
+    for lib in (L, T):
+        o, dq, dk, dv = (torch.full_like(q, float("nan")) for _ in range(4))
+        lse = torch.empty(B, H, M, device=dev, dtype=torch.float32)
+        delta = torch.empty_like(lse)
+        plan = _Plan(q, k, v, True, 1.0 / math.sqrt(D), ids, ids, 1)
+        p = plan.p
+        p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+            _set4(getattr(p, f), t)
+        plan.ensure_workspace(dev)
+        p.flags = _cabi.FA_FLAG_DQ_DELTA
+        ref, stream = ctypes.byref(p), _stream_ptr(dev)
+        for name in ("fa_mask_plan", "fa_fwd", "fa_bwd_dq", "fa_bwd_dkdv"):
+            fn = getattr(lib, name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.POINTER(_cabi.FaParams), ctypes.c_void_p]
+            assert fn(ref, stream) == 0, name
+        torch.cuda.synchronize()
+        results.append((o, lse, dq, dk, dv))
+    for a_, b_ in zip(*results):
+        assert not torch.isnan(a_).any() and torch.equal(a_, b_)
+
+
 def test_empty_inputs():
     """No query rows, no batch, or no keys at all: nothing is launched; O has q's shape (zeros where there are
     rows: a row without keys behaves as a row whose keys are all masked, O = 0 and LSE = -inf) and the
