@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 6
+#define FA_ABI_VERSION 7
 
 /* score_func_mode, flash_triton.py:20-22 */
 #define FA_SCORE_MODE0_NOPE 0
@@ -92,7 +92,9 @@ extern "C" {
                                has used a P it cannot trust and REPORTS it by writing NaN into its 32 rows of dk
                                (dv is not affected).  A NaN in dk after a backward with finite inputs therefore
                                means "a pair wait expired", not an arithmetic overflow.  With this flag the poll
-                               budget is zero, so the report can be provoked without hanging or faulting anything. */
+                               budget is zero, so the report can be provoked without hanging or faulting anything.
+                               Accepted by fa_bwd_dkdv only; every other entry point refuses it (FA_ERR_MODE).
+                               Every expiry is also counted, see fa_pair_wait_expired. */
 
 typedef struct fa_params {
   /* forward operands */
@@ -145,6 +147,15 @@ typedef struct fa_params {
      stores the positions with the plan), and by fa_mask_dump. */
   const int32_t* qpos;
   int64_t qpos_stride;    /* batch stride of qpos in elements (0: one vector for every batch) */
+  /* Optional home of the stateless part of the workspace (the partial results of key ranges that are
+     split over several workgroups), so that a caller can keep the small plan between forward and
+     backward -- as the reference keeps eq / ek in its ctx, flash_triton.py:557-562 -- without holding
+     on to, copying or re-planning anything else.  NULL: that part follows the plan inside `workspace`
+     (which then needs fa_workspace_bytes).  Non-NULL (256-byte aligned, at least
+     fa_workspace_scratch_bytes): `workspace` needs fa_workspace_plan_bytes only.  Nothing is carried in
+     it from one call to the next; two launches that share it must be ordered on one stream. */
+  void*       split_scratch;
+  uint64_t    split_scratch_bytes;
 } fa_params;
 
 /* ABI version of the loaded library (== FA_ABI_VERSION of the header it was built from). */
@@ -161,7 +172,8 @@ int fa_last_hip_error(void);
 
 /* Shape / dtype / stride / alignment / null checks for the given stage.
    Touches no GPU API; callable on a machine without a GPU.
-   stage: 0 = forward, 1 = backward (all three backward kernels), 2 = mask plan only. */
+   stage: 0 = forward, 1 = backward (fa_bwd_delta, fa_bwd_dq), 2 = mask plan only,
+          3 = fa_bwd_dkdv (stage 1, and FA_FLAG_DEBUG_NO_PAIR_WAIT is accepted). */
 int fa_validate(const fa_params* p, int stage);
 
 /* Bytes of workspace fa_mask_plan needs for these sizes (0 when score_mode == 0). */
@@ -172,6 +184,10 @@ uint64_t fa_workspace_bytes(const fa_params* p);
    A caller that keeps a plan between forward and backward (as the reference keeps eq/ek,
    flash_triton.py:557) needs to keep this prefix only and may copy it into a fresh workspace. */
 uint64_t fa_workspace_plan_bytes(const fa_params* p);
+
+/* Bytes of the stateless rest (what p->split_scratch may carry instead of the tail of the workspace);
+   fa_workspace_bytes = plan bytes + scratch bytes.  0 when no key range of these sizes is ever split. */
+uint64_t fa_workspace_scratch_bytes(const fa_params* p);
 
 /* Mask engine: normalise eq/ek to int32 and build per-tile id summaries
    into p->workspace.  Must be enqueued before fa_fwd / fa_bwd_* on the same
@@ -209,6 +225,12 @@ int fa_bwd_dkdv(const fa_params* p, void* stream);
 
 /* dq (needs lse, and delta unless FA_FLAG_DQ_DELTA is set). */
 int fa_bwd_dq(const fa_params* p, void* stream);
+
+/* Number of wave-level pair waits of fa_bwd_dkdv that expired on the current device since the library
+   was loaded (see FA_FLAG_DEBUG_NO_PAIR_WAIT: each one also shows as NaN in 32 rows of dk).  0 in any
+   healthy run.  Waits for the device to be idle before it reads the count (a diagnostic, not for hot
+   loops); returns FA_OK or FA_ERR_HIP.  No counterpart in the reference. */
+int fa_pair_wait_expired(uint64_t* count);
 
 /* Write keep(i,j) as one byte (0/1) per element into out[B,H,M,N] (contiguous),
    evaluated by the same device routine the compute kernels use. */

