@@ -33,6 +33,17 @@ def plan_q(eq, M, pos=None):
     return perm, hdr, sums
 
 
+def first_local_key_tile(qsums, ksums, causal, gap):
+    """Header field k0: the first key tile that any summary entry of local rows visits (INT_MAX: none)."""
+    k0 = INT_MAX
+    for s in qsums:
+        if s["nvalid"] and not s["glob"]:
+            cand = [kt for kt, k_ in enumerate(ksums) if visits(s, k_, kt, causal, gap)]
+            if cand:
+                k0 = min(k0, cand[0])
+    return k0
+
+
 def plan_k(ek, N):
     sums = []
     for t in range((N + SUM - 1) // SUM):

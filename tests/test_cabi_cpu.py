@@ -124,7 +124,7 @@ def test_workspace_size():
     p.ek_stride[0], p.ek_stride[1], p.ek_stride[2] = 4 * 256, 256, 1   # per head
     r256 = lambda x: (x + 255) // 256 * 256
     Pp = 256 + 256
-    want = (r256(128 * 4) + r256(4 * 256 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+    want = (r256(128 * 4) + r256(4 * 256 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(32) + r256(Pp // 64 * 32)
             + r256(4 * 4 * 32))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want   # 4 key tiles of 64: no key range is ever split
     assert L.fa_workspace_plan_bytes(ctypes.byref(p)) == want   # ... so all of it is plan
@@ -135,7 +135,7 @@ def test_workspace_size():
     p.ek_stride[0], p.ek_stride[1] = 4 * 2048, 2048
     chunks, tiles = 2, 2   # 32 key tiles -> 2 chunks of 16; M = 128 rows -> 2 tiles
     assert p.M == 128 and (128 << 20) // (1 * 4 * chunks * 128 * (p.D + 2) * 4) >= 64
-    want = (r256(128 * 4) + r256(4 * 2048 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(16) + r256(Pp // 64 * 32)
+    want = (r256(128 * 4) + r256(4 * 2048 * 4) + 3 * r256(Pp * 4) + r256(4) + r256(32) + r256(Pp // 64 * 32)
             + r256(4 * 32 * 32)
             + r256(4 * tiles * 4) + r256(4 * tiles * chunks * 128 * 2 * 4) + r256(4 * tiles * chunks * 128 * p.D * 4))
     assert L.fa_workspace_bytes(ctypes.byref(p)) == want

@@ -693,7 +693,7 @@ def test_device_mask_plan_matches_host_restatement():
     o_pq = off; off += r256(B * H * Pp * 4)
     o_pp = off; off += r256(B * H * Pp * 4)
     off += r256(B * H * ((Mp + 1023) // 1024) * 4)     # per-chunk counts of the partition
-    o_hd = off; off += r256(B * H * 16)
+    o_hd = off; off += r256(B * H * 32)
     o_qs = off; off += r256(B * H * nQs * 32)
     o_ks = off; off += r256(B * H * nKs * 32)
     # no scratch for split tiles here: N / 64 < 32 key tiles, no key range is ever cut
@@ -703,7 +703,7 @@ def test_device_mask_plan_matches_host_restatement():
     peq = i32(o_pq, B * H * Pp).reshape(B, H, Pp)
     ppos = i32(o_pp, B * H * Pp).reshape(B, H, Pp)
     assert np.array_equal(ppos, np.where(perm >= 0, perm + (N - M), -1))   # diagonal positions: gap + row
-    hdr = i32(o_hd, B * H * 4).reshape(B, H, 4)
+    hdr = i32(o_hd, B * H * 8).reshape(B, H, 8)
     qs = i32(o_qs, B * H * nQs * 8).reshape(B, H, nQs, 8)
     ks = i32(o_ks, B * H * nKs * 8).reshape(B, H, nKs, 8)
     assert np.array_equal(i32(o_eq, B * H * Mp).reshape(B, H, Mp)[:, :, :M], eq)
@@ -714,7 +714,8 @@ def test_device_mask_plan_matches_host_restatement():
             assert np.array_equal(perm[b, h], rp)
             assert np.array_equal(peq[b, h][rp >= 0], eq[b, h][rp[rp >= 0]])
             rk = P.plan_k(ek[b, h].astype(np.int64), N)
-            assert list(hdr[b, h]) == [rh["nL"], rh["nG"], rh["nLp"], rh["nT128"]]
+            assert list(hdr[b, h][:4]) == [rh["nL"], rh["nG"], rh["nLp"], rh["nT128"]]
+            assert hdr[b, h][4] == P.first_local_key_tile(rq, rk, True, N - M)
             for t, s_ in enumerate(rq):
                 got = qs[b, h, t]
                 # the device stores key positions of the rows' diagonals: gap + row without per-row positions
@@ -813,6 +814,32 @@ def test_varlen_takes_boundaries_from_the_host_and_needs_key_boundaries_for_othe
     assert torch.equal(attention_varlen(q, q, q, cuq), attention_varlen(q, q, q, cuq.cuda()))
     with pytest.raises(AssertionError, match="cu_seqlens_k"):
         attention_varlen(q, k, v, cuq.cuda())
+
+
+COLS_CASES = [
+    # B, H, Hk, M, N, D, dtype, causal, ids, window: more keys than queries, the queries' documents at the end
+    (2, 2, 2, 300, 1500, 128, torch.bfloat16, True, "uniform", 0),     # one tile of global rows
+    (1, 4, 2, 300, 1700, 128, torch.float16, True, "uniform", 0),      # grouped heads: one tile per query head
+    (1, 2, 2, 900, 2100, 128, torch.bfloat16, True, "uniform", 0),     # two tiles
+    (1, 2, 2, 2000, 3100, 128, torch.bfloat16, True, "uniform", 0),    # three tiles: the general kernel keeps these columns
+    (1, 2, 2, 300, 1500, 128, torch.bfloat16, True, "alllocal", 0),    # no global row at all: the columns get zeros
+    (1, 2, 2, 300, 1501, 64, torch.float16, True, "uniform", 0),       # ragged key count, D = 64
+    (2, 2, 1, 200, 1333, 16, torch.bfloat16, True, "uniform", 0),
+    (1, 2, 2, 333, 1777, 32, torch.bfloat16, True, "uniform", 0),
+    (1, 2, 2, 300, 1500, 128, torch.bfloat16, True, "uniform", 700),   # sliding window: global rows lose the far keys
+    (1, 2, 2, 300, 1500, 128, torch.bfloat16, False, "uniform", 0),    # no causal mask
+    (1, 2, 2, 64, 4100, 128, torch.bfloat16, True, "allglobal", 0),    # every row global: all key columns
+]
+
+
+@pytest.mark.parametrize("case", COLS_CASES, ids=lambda c: "B%d-H%d_%d-M%d-N%d-D%d-%s-c%d-%s-w%d" % (
+    c[0], c[1], c[2], c[3], c[4], c[5], str(c[6]).split(".")[-1], c[7], c[8], c[9]))
+def test_key_columns_that_only_global_rows_see(case):
+    """dK / dV of key columns no local row can need come from a kernel of their own (the global rows'
+    Q / dO tiles resident, the keys streamed) when the global rows are few; the other columns and every
+    other shape stay with the general kernel.  Both against the oracle, and the seam between them."""
+    B, H, Hk, M, N, D, dtype, causal, kind, window = case
+    _run_case(B, H, Hk, M, N, D, dtype, causal, True, seed=77 + M + N, ids_kind=kind, window=window)
 
 
 def test_delta_with_more_than_65535_batch_head_pairs():

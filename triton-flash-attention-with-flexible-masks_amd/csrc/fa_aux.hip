@@ -144,6 +144,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(int M, int Mp, int Pp
   if (ch == 0 && tid == 0) {
     QHeader q;
     q.nL = nL; q.nG = nG; q.nLp = nLp; q.nT128 = (nLp + (nG + 127) / 128 * 128) / 128;
+    q.k0 = 0x7fffffff; q.pad[0] = q.pad[1] = q.pad[2] = 0;   // k0: lowered by plan_qsum_kernel
     hdr[bh] = q;
   }
 }
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs
                                                         const int* __restrict__ perm, const int* __restrict__ peq,
                                                         const int* __restrict__ ppos,
                                                         const IdSummary* __restrict__ ksum, IdSummary* __restrict__ qsum,
-                                                        int* __restrict__ sk_cnt, int n_sk) {
+                                                        int* __restrict__ sk_cnt, int n_sk, QHeader* __restrict__ hdr) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // the arrival counters of the split-key merge start every forward at zero
   if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)
@@ -198,7 +199,11 @@ __global__ __launch_bounds__(256) void plan_qsum_kernel(int Pp, int nQs, int nKs
   }
   s.kfirst = s.nvalid > 0 ? kfirst : 0x7fffffff;
   s.klast = s.nvalid > 0 ? klast : -1;
-  if (lane == 0) qsum[bh * nQs + t] = s;
+  if (lane == 0) {
+    qsum[bh * nQs + t] = s;
+    // first key tile any local row can need (the header starts at "none", set by plan_scatter_kernel)
+    if (s.nvalid > 0 && s.glob == 0) atomicMin(&hdr[bh].k0, s.klast >= s.kfirst ? s.kfirst : 0x7fffffff);
+  }
 }
 
 int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
@@ -237,7 +242,7 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     hipLaunchKernelGGL(plan_qsum_kernel, dim3((w.nQs + 3) / 4, w.Hq1, p->B), dim3(256), 0, s, w.Pp, w.nQs, w.nKs, w.Hq1, w.Hk1,
                        p->causal ? 1 : 0, p->prefix > 0 ? ((p->prefix < p->N ? p->prefix : p->N) - 1) / kSumRows + 1 : 0, perm, peq, ppos, ksum, qsum, reinterpret_cast<int*>(ws + w.off_sk_cnt),
-                       p->B * p->H * w.split.tiles);
+                       p->B * p->H * w.split.tiles, hdr);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   return 0;

@@ -29,6 +29,8 @@ namespace fa {
 constexpr int kKvPre = 4;
 constexpr int kKvPre2 = 3;
 
+constexpr int kColsRun = 8;   // key tiles per workgroup when the column form shares the launch
+
 // SPLIT = true : two waves per block of 32 keys, NKB key blocks per workgroup, roles split over the
 //                wave pairs as described above (D = 128: one wave cannot hold both operand sets and
 //                both accumulator sets next to a second wave on its SIMD).
@@ -44,8 +46,17 @@ __device__ unsigned long long g_pair_expired = 0;
 FA_TRACE_ARRAY(g_trace_dkdv);
 #endif
 
-template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT, int NKB>
-__global__ __launch_bounds__(SPLIT ? 128 * NKB : 64 * NKB) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 3 : 2, D <= 32 ? 3 : 2)))
+}  // namespace fa
+#include "fa_dkdv_cols.h"   // the column form; its workgroups stamp the same array: 0 start, 3 tiles resident, 4 after the key loop, 5 end, 6 key blocks of wave 0, 7 chunk | 1 << 40
+namespace fa {
+
+// COLS = true : the grid carries, behind the workgroups of this form, those of the column form
+//                (fa_dkdv_cols.h) for the leading key columns that only a few global rows see; the workgroups
+//                of this form whose keys lie there leave at once.  One launch, so the column form's memory
+//                traffic overlaps the set-up latencies of this one.
+template <typename Tag, int D, bool CAUSAL, bool DOC, bool SPLIT, int NKB, bool COLS>
+__global__ __launch_bounds__(SPLIT ? 128 * NKB : 64 * NKB)
+__attribute__((amdgpu_waves_per_eu((D <= 32 && !COLS) ? 3 : 2, (D <= 32 && !COLS) ? 3 : 2)))
 void bwd_dkdv_kernel(const KArgs a) {
   using E = Elem<Tag>;
   using T = typename E::scalar;
@@ -68,6 +79,21 @@ void bwd_dkdv_kernel(const KArgs a) {
   static_assert(NW >= 4, "the four auxiliary arrays of a tile are loaded by waves 0..3");
   using Loader = TileLoader<DL, BQ, D, NW>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int nKt = (a.N + BK - 1) / BK;
+  // With the column form in the launch, most key tiles of this form may have nothing to do here (their keys
+  // belong to the column form): a workgroup then takes kColsRun key tiles, nSlots tiles apart, and steps over
+  // those -- a workgroup that only finds out that it is not needed costs the dispatcher as much as a short
+  // useful one (8192 of them: 50 us), a skipped tile of a run costs a comparison.
+  const int nSlots = COLS ? (nKt + kColsRun - 1) / kColsRun : nKt;
+  int bid = (int)blockIdx.x;   // index of the workgroup among those of its form
+  if constexpr (COLS) {
+    static_assert(DOC && (SPLIT ? 128 * NKB : 64 * NKB) == 256, "the column form runs with ids, 4 waves per workgroup");
+    // the column form's workgroups come first: few, long, one round of them
+    const int nC = dkdv_cols_blocks(a);
+    const bool cols = bid < nC;
+    if (!cols) bid -= nC;
+    if (cols) { dkdv_cols_body<Tag, D, CAUSAL>(a, bid, smem); return; }
+  }
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar
   const int role = SPLIT ? wave / NKB : 0, kb = wave % NKB;
@@ -75,13 +101,19 @@ void bwd_dkdv_kernel(const KArgs a) {
   FA_STAMP(g_trace_dkdv, 0, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 5, 0); FA_STAMP(g_trace_dkdv, 7, -1);
   FA_TRACE_ONLY(int tr_tiles = 0; bool tr_first = false; long long tr_wait = 0;)
 
-  // one workgroup per (key tile, batch, kv head)
-  const int nKt = (a.N + BK - 1) / BK;
-  int kt, bhk;
-  if (!block_to_tile(nKt, a.B * a.Hk, false, kt, bhk)) return;  // causal: the first key tiles see the most rows
+  // one workgroup per (key tile, batch, kv head) -- or per run of key tiles, see above
+  int kt0, bhk;
+  if (!block_to_tile(nSlots, a.B * a.Hk, false, kt0, bhk, bid)) return;  // causal: the first key tiles see the most rows
   const int b = bhk / a.Hk, hk = bhk % a.Hk;
-
+  const int ncols = COLS ? gcol_info(a, b, hk).ncols : 0;   // leading keys that belong to the column form of this launch
+  bool ran = false;
+  for (int rr = 0; rr < (COLS ? kColsRun : 1); ++rr) {
+  const int kt = kt0 + rr * nSlots;
   const int n0 = kt * BK;
+  if (COLS && (kt >= nKt || n0 + BK <= ncols)) continue;
+  if (COLS && ran) __syncthreads();   // the previous key tile's last reads of LDS are done
+  ran = true;
+  pair_lost = 0;
   const int nw = n0 + kb * 32;
   const int key = nw + lq;
   const int keyc = key < a.N ? key : a.N - 1;
@@ -635,21 +667,24 @@ void bwd_dkdv_kernel(const KArgs a) {
       store(dkrow, acc2, a.scale);
     }
   }
+  }   // run of key tiles
   FA_STAMP(g_trace_dkdv, 5, FA_CLOCK());
 }
 
 // Query tiles per workgroup (no ids) below which the 64-key role-split form is launched.
 constexpr int kKvShortTiles = 32;
-template <typename Tag, int D, bool CAUSAL, bool DOC, int NKB>
+template <typename Tag, int D, bool CAUSAL, bool DOC, int NKB, bool COLS = false>
 static int launch_nkb(const KArgs& a, hipStream_t s) {
   constexpr bool SPLIT = D > 64;
   constexpr int BK = 32 * NKB, BQ = 64;
   const int nKt = (a.N + BK - 1) / BK;
-  const size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 + 64 : 0);
-  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT, NKB>;
+  size_t lds = 4 * BQ * (D < 32 ? 32 : D) * 2 + 2 * 1024 + (SPLIT ? 2 * NKB * 2048 + 64 : 0);
+  if (COLS && dkdv_cols_lds(D) > lds) lds = dkdv_cols_lds(D);
+  auto kern = bwd_dkdv_kernel<Tag, D, CAUSAL, DOC, SPLIT, NKB, COLS>;
   static bool lds_allowed[64] = {};   // per kernel instantiation and device
   if (int e = allow_lds(kern, lds, lds_allowed)) return e;
-  hipLaunchKernelGGL(kern, dim3(grid_blocks(nKt, a.B * a.Hk)), dim3(SPLIT ? 128 * NKB : 64 * NKB), lds, s, a);
+  const int blocks = COLS ? grid_blocks((nKt + kColsRun - 1) / kColsRun, a.B * a.Hk) + dkdv_cols_blocks(a) : grid_blocks(nKt, a.B * a.Hk);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(SPLIT ? 128 * NKB : 64 * NKB), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -663,6 +698,13 @@ static int launch_one(const KArgs& a, hipStream_t s) {
   // causal mask, at most a window's worth under a sliding window.  Under a block mask the 64-key
   // form is one column of blocks: no wave waits at a tile that only the other column needs
   // (diagonal + 25 % random blocks at 16K tokens: 1.81 -> 1.24 ms).
+  // A key prefix without a diagonal of its own (more keys than queries), per-row positions or no causal
+  // mask at all: local rows may need none of the leading keys, and the column form takes those (it decides
+  // on the device, from the mask plan, how many they are -- possibly none).  Square causal problems with the
+  // same ids on both sides always have a local row on the first keys' diagonal: nothing to gain there.
+  if constexpr (DOC) {
+    if (a.gap >= kGcolMinGap || a.qpos != nullptr || !CAUSAL) return launch_nkb<Tag, D, CAUSAL, DOC, (D > 64 ? 2 : 4), true>(a, s);
+  }
   if constexpr (D > 64) {
     if (DOC || a.bmask != nullptr) return launch_nkb<Tag, D, CAUSAL, DOC, 2>(a, s);
     int tiles = (a.M + 63) / 64;

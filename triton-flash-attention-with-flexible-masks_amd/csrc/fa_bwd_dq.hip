@@ -87,8 +87,11 @@ void bwd_dq_kernel(const KArgs a) {
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
   QBlockMask bmq;
   bmq.init(a, b, h, wk.tile);
+  const bool halved = qc.halved;
+  const int sub = __builtin_amdgcn_readfirstlane(qc.sub);   // halved tiles (QTileCtx): this wave computes keys 32 * sub .. of every key tile
   auto dec = [&](int t, const IdSummary& ks) {
-    return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi) | (DOC ? 0 : bmq.flags(t)), 0);
+    const int fl = halved ? qc.decide(a, t * BN + 32 * sub, 32, ks.lo, ks.hi) : qc.decide(a, t * BN, BN, ks.lo, ks.hi);
+    return tile_value(fl | (DOC ? 0 : bmq.flags(t)), 0);
   };
   TileIter it;
   it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);   // its summaries travel together with Q, dO
@@ -106,7 +109,7 @@ void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) part += float(of[ks][t]) * float(dof[ks][t]);
     delta_i = xhalf_sum(part);
-    if (row >= 0 && g == 0 && wk.split == 0) delp[row] = delta_i;   // for the dk/dv kernel
+    if (row >= 0 && g == 0 && wk.split == 0 && sub == 0) delp[row] = delta_i;   // for the dk/dv kernel
   }
   if (L_i == -INFINITY) L_i = INFINITY;  // row without any kept key: P = exp2(-inf) = 0
 
@@ -115,6 +118,15 @@ void bwd_dq_kernel(const KArgs a) {
   ldV.init(vp, a.v_rs, a.N);
   LdsOffsets<DL> lo;
   lo.init();
+  int id_off = g * 16, key_off = 0;
+  if (halved) {   // this wave's half of every key tile
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) lo.row[ks] += sub * (32 * DL * 2);
+#pragma unroll
+    for (int db = 0; db < DBN; ++db) { lo.tr[db][0] += sub * (32 * DL * 2); lo.tr[db][1] += sub * (32 * DL * 2); }
+    id_off += sub * (32 * 4);
+    key_off = 32 * sub;
+  }
 
   f32x16 dq[DBN];
 #pragma unroll
@@ -125,13 +137,13 @@ void bwd_dq_kernel(const KArgs a) {
   auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
-    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
-    const int n0 = cur * BN;
+    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + id_off;  // the tile's key ids
+    const int n0 = cur * BN + key_off;
     if (flags & TF_SKIP) return;
     const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    // one 32-key block of the tile (kb a literal on the usual path: every offset an immediate)
+    auto block = [&](const int kb) __attribute__((always_inline)) {
       f32x16 s = zero, dp = zero;
       __builtin_amdgcn_sched_barrier(0);
       // S and dP are accumulated alternately (an MFMA that accumulates onto the result of the MFMA
@@ -200,7 +212,9 @@ void bwd_dq_kernel(const KArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-    }
+    };
+    block(0);
+    if (!halved) block(1);   // (halved tiles: the lane offsets point into this wave's half, which is its whole tile)
   };
 
   // tile streams: K, V and (with ids) the 64 key ids of the tile, all straight into LDS
@@ -233,17 +247,37 @@ void bwd_dq_kernel(const KArgs a) {
   }
   FA_STAMP(g_trace_dq, 3, FA_CLOCK()); FA_STAMP(g_trace_dq, 5, tr_tiles);
 
+  if (halved) {
+    // the wave that took the second half of every key tile hands its partial dQ to the wave that took the
+    // first half of the same rows, lane for lane, through the LDS the tile stream no longer needs
+    __syncthreads();   // every wave is done with the last tile
+    float* mb = reinterpret_cast<float*>(smem) + qc.rb * (16 * DBN * 64) + lane;
+    if (sub == 1) {
+#pragma unroll
+      for (int db = 0; db < DBN; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mb[(16 * db + r) * 64] = dq[db][r];
+    }
+    __syncthreads();
+    if (sub == 0) {
+#pragma unroll
+      for (int db = 0; db < DBN; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq[db][r] += mb[(16 * db + r) * 64];
+    }
+  }
+  const bool writer = !halved || sub == 0;   // the wave that holds the rows' result
   if (DOC && nsplit > 1) {
     // This workgroup saw one chunk of the keys: store the partial sum; the last chunk to arrive
     // adds them up in a fixed order and writes dQ.
     const int64_t tbase = (int64_t(b) * a.H + h) * a.split_tiles + wk.gt;
     float* po = a.sk_o + (tbase * a.split_k + wk.split) * (128 * D);
-    const int rt = (threadIdx.x >> 6) * 32 + (lane & 31);   // row inside the tile
+    const int rt = qc.rb * 32 + (lane & 31);   // row inside the tile
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        if (32 * db + 8 * q4 >= D) continue;
+        if (32 * db + 8 * q4 >= D || !writer) continue;
         f32x4 x = {dq[db][4 * q4 + 0], dq[db][4 * q4 + 1], dq[db][4 * q4 + 2], dq[db][4 * q4 + 3]};
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
@@ -307,7 +341,7 @@ void bwd_dq_kernel(const KArgs a) {
     return;
   }
 
-  if (row >= 0) {
+  if (row >= 0 && writer) {
     T* drow = dqp + int64_t(row) * a.dq_rs;
     const float sc = a.scale;
 #pragma unroll

@@ -242,6 +242,9 @@ struct IdSummary {
 
 struct QHeader {
   int nL, nG, nLp, nT128;  // nT128: 128-row tiles of the permuted order that hold rows
+  int k0;                  // first key tile (of 64) that a local row can need (0x7fffffff: none can need any):
+                           // the keys before it are seen by global rows only
+  int pad[3];
 };
 
 // A tile pair can hold a kept element only if a global query row exists or the
@@ -254,6 +257,13 @@ FA_DEV bool doc_all_keep(int q_lo, int q_hi, int k_lo, int k_hi) {
   // no local row at all, or one local id shared by every key
   return (q_lo > q_hi) || (q_lo == q_hi && k_lo == k_hi && q_lo == k_lo);
 }
+
+// Key columns that no local row can need (QHeader::k0) are seen by the global rows only.  When those rows
+// are few -- at most kGcolTilesMax tiles of 64, over all query heads of a group -- a kernel of its own takes
+// these columns: it keeps the rows' Q / dO tiles in LDS and streams the keys (fa_dkdv_cols.h), instead
+// of one workgroup per 64 keys that sets up a tile stream for one or two tiles.
+constexpr int kGcolTilesMax = 2;
+constexpr int kGcolMinGap = 512;   // keys without a diagonal of their own from which the form is put into the launch
 
 // Kernel-side view of the operands (built on the host from fa_params).
 struct KArgs {

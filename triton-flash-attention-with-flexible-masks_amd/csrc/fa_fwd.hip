@@ -88,8 +88,11 @@ void fwd_kernel(const KArgs a) {
   // decisions of this wave for key tile t, evaluated by the lane that tests the tile
   QBlockMask bmq;
   bmq.init(a, b, h, wk.tile);
+  const bool halved = qc.halved;
+  const int sub = __builtin_amdgcn_readfirstlane(qc.sub);   // halved tiles: this wave computes keys 32 * sub .. of every key tile
   auto dec = [&](int t, const IdSummary& ks) {
-    return tile_value(qc.decide(a, t * BN, BN, ks.lo, ks.hi) | (DOC ? 0 : bmq.flags(t)), 0);
+    const int fl = halved ? qc.decide(a, t * BN + 32 * sub, 32, ks.lo, ks.hi) : qc.decide(a, t * BN, BN, ks.lo, ks.hi);
+    return tile_value(fl | (DOC ? 0 : bmq.flags(t)), 0);
   };
   TileIter it;
   it.init_keys(kt_first, kt_last, qc.ksum, qc.g_lo, qc.g_hi, qc.g_glob, dec);   // its summaries travel together with Q
@@ -110,6 +113,15 @@ void fwd_kernel(const KArgs a) {
   ldV.init(vp, a.v_rs, a.N);
   LdsOffsets<DL> lo;
   lo.init();
+  int id_off = g * 16, key_off = 0;
+  if (halved) {   // this wave's half of every key tile
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) lo.row[ks] += sub * (32 * DL * 2);
+#pragma unroll
+    for (int db = 0; db < DBN; ++db) { lo.tr[db][0] += sub * (32 * DL * 2); lo.tr[db][1] += sub * (32 * DL * 2); }
+    id_off += sub * (32 * 4);
+    key_off = 32 * sub;
+  }
 
   f32x16 o[DBN];
 #pragma unroll
@@ -123,36 +135,45 @@ void fwd_kernel(const KArgs a) {
   float l_run = 0.f;        // this lane's partial row sum
 
   // One K/V tile; BUF is a compile-time constant so every LDS address is base + immediate.
-  auto compute = [&](const int BUF, const int cur, const int flags) __attribute__((always_inline)) {
+  // nb_c: 32-key blocks of the tile this wave computes: both, or (halved tiles, see QTileCtx) one -- the lane
+  // offsets `lo`, `id_off` and `key_off` then point into that block, so both forms use the same immediates.
+  auto compute = [&](const int BUF, const int cur, const int flags, auto nb_c) __attribute__((always_inline)) {
+    constexpr int NB = decltype(nb_c)::value;
     const char* lk = smem + BUF * TILE_BYTES;
     const char* lv = smem + (2 + BUF) * TILE_BYTES;
-    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + g * 16;  // the tile's key ids
-    const int n0 = cur * BN;
+    const char* lid = smem + 4 * TILE_BYTES + BUF * (BN * 4) + id_off;  // the tile's key ids
+    const int n0 = cur * BN + key_off;
 
     if (flags & TF_SKIP) return;
     const bool need_lim = (flags & TF_LIM) != 0, need_doc = (flags & TF_DOC) != 0;
 
     f32x16 s[2];
     __builtin_amdgcn_sched_barrier(0);
-    // The two 32-key blocks are accumulated alternately: an MFMA that accumulates onto the result
-    // of the MFMA issued right before it waits a full extra MFMA time, two interleaved chains do not.
+    // Two accumulator chains are fed alternately: an MFMA that accumulates onto the result of the MFMA
+    // issued right before it waits a full extra MFMA time, two interleaved chains do not.  With both
+    // blocks the chains are the blocks; with one block they are its even and odd k-steps, added up after.
     {
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       s[0] = zero;
       s[1] = zero;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
+        if constexpr (NB == 2) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
-          s[kb] = E::mfma32(kf, qf[ks], s[kb]);
+          for (int kb = 0; kb < 2; ++kb) {
+            const vec8 kf = lds_row8<E>(lk + lo.row[ks] + kb * 32 * DL * 2);
+            s[kb] = E::mfma32(kf, qf[ks], s[kb]);
+          }
+        } else {
+          const vec8 kf = lds_row8<E>(lk + lo.row[ks]);
+          s[ks & 1] = E::mfma32(kf, qf[ks], s[ks & 1]);
         }
       }
     }
     // Instruction order of this region: keep several K fragments in flight ahead of the MFMA that
     // consumes them (an LDS read takes about as long as three MFMAs).
     {
-      constexpr int NQK = 2 * KS, PRE = NQK < kFwdPre ? NQK : kFwdPre;
+      constexpr int NQK = NB * KS, PRE = NQK < kFwdPre ? NQK : kFwdPre;
       __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
       for (int i = 0; i < NQK - PRE; ++i) {
@@ -162,17 +183,23 @@ void fwd_kernel(const KArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x008, PRE, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NB == 1) {
+      if (KS > 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[0][r] += s[1][r];
+      }
+    }
     if (need_lim) {
       asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: never if-converted
       const int rel = qc.lim_i - n0 - 4 * g;
       const int rel_lo = qc.low_i - n0 - 4 * g;
       mask_lim(s[0], rel, rel_lo, -INFINITY);
-      mask_lim(s[1], rel - 32, rel_lo - 32, -INFINITY);
+      if constexpr (NB == 2) mask_lim(s[1], rel - 32, rel_lo - 32, -INFINITY);
     }
     if (DOC && need_doc) {
       asm volatile("" ::: "memory");
       mask_doc(s[0], lid, eq_i, qc.glob_i, -INFINITY);
-      mask_doc(s[1], lid + 32 * 4, eq_i, qc.glob_i, -INFINITY);
+      if constexpr (NB == 2) mask_doc(s[1], lid + 32 * 4, eq_i, qc.glob_i, -INFINITY);
     }
     // Online softmax in the exp2 domain with a lazily moved reference point.  Fast path: the
     // exponentials are taken against the reference point as it stands and only their sum is looked
@@ -182,24 +209,34 @@ void fwd_kernel(const KArgs a) {
     // whole wave through the full path: row maximum, new reference point, O and l rescaled.  A row
     // that has not met a kept key yet stays on the fast path (its exponentials are exact zeros).
     constexpr float kSumLimit = 4096.f;   // per lane over its 32 keys: every p <= 4096 (fits fp16 too)
-    f32x16 p[2];
+    f32x16 p[NB];
     float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -m_ref));
-      p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -m_ref));
       ps0 += p[0][r];
-      ps1 += p[1][r];
+      if constexpr (NB == 2) {
+        p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -m_ref));
+        ps1 += p[1][r];
+      }
     }
     if (__builtin_amdgcn_ballot_w64(!(ps0 + ps1 <= kSumLimit)) != 0) {
-      float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
-      float mx1 = fmaxf(fmaxf(s[1][0], s[1][1]), s[1][2]);
+      float mx;
+      if constexpr (NB == 2) {
+        float mx0 = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
+        float mx1 = fmaxf(fmaxf(s[1][0], s[1][1]), s[1][2]);
 #pragma unroll
-      for (int r = 3; r < 15; r += 2) {
-        mx0 = fmaxf(fmaxf(mx0, s[0][r]), s[0][r + 1]);
-        mx1 = fmaxf(fmaxf(mx1, s[1][r]), s[1][r + 1]);
+        for (int r = 3; r < 15; r += 2) {
+          mx0 = fmaxf(fmaxf(mx0, s[0][r]), s[0][r + 1]);
+          mx1 = fmaxf(fmaxf(mx1, s[1][r]), s[1][r + 1]);
+        }
+        mx = fmaxf(fmaxf(mx0, mx1), fmaxf(s[0][15], s[1][15]));
+      } else {
+        mx = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, s[0][r]), s[0][r + 1]);
+        mx = fmaxf(mx, s[0][15]);
       }
-      float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(s[0][15], s[1][15]));
       mx = xhalf_max(mx) * c;   // -inf stays -inf (c > 0)
       {
         // the reference point moves to the running maximum whenever this path is taken (after it
@@ -218,19 +255,24 @@ void fwd_kernel(const KArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         p[0][r] = fast_exp2(__builtin_fmaf(s[0][r], c, -msub));
-        p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -msub));
         ps0 += p[0][r];
-        ps1 += p[1][r];
+        if constexpr (NB == 2) {
+          p[1][r] = fast_exp2(__builtin_fmaf(s[1][r], c, -msub));
+          ps1 += p[1][r];
+        }
       }
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { s[0][r] = p[0][r]; s[1][r] = p[1][r]; }
+    for (int r = 0; r < 16; ++r) {
+      s[0][r] = p[0][r];
+      if constexpr (NB == 2) s[1][r] = p[1][r];
+    }
     l_run += ps0 + ps1;
     // O^T += V^T P^T, 16 keys per MFMA.  V^T fragments (two transposed reads each) are requested
     // PRE MFMAs ahead in program order, P is converted just in time; the scheduling barriers pin
     // that order (left to itself the scheduler puts every read right before its MFMA).
     {
-      constexpr int NPV = 4 * DBN, PRE = NPV < kFwdPre2 ? NPV : kFwdPre2;
+      constexpr int NPV = 2 * NB * DBN, PRE = NPV < kFwdPre2 ? NPV : kFwdPre2;
       auto fetch = [&](const int i) __attribute__((always_inline)) {
         const int c16 = i / DBN, db = i % DBN;
         return lds_tr8<E>(lv + lo.tr[db][0] + c16 * 16 * DL * 2, lv + lo.tr[db][1] + c16 * 16 * DL * 2);
@@ -269,25 +311,57 @@ void fwd_kernel(const KArgs a) {
   int cur_fl = it.flags;
   FA_STAMP(g_trace_fwd, 2, FA_CLOCK());
   if (cur >= 0) issue(0, cur);
-  while (cur >= 0) {
-    int nxt = it.next(dec);
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) issue(1, nxt);
-    compute(0, cur, cur_fl);
-    FA_TRACE_ONLY(++tr_tiles;)
-    cur = nxt; cur_fl = it.flags;
-    if (cur < 0) break;
-    nxt = it.next(dec);
-    wait_async_loads();
-    __syncthreads();
-    if (nxt >= 0) issue(0, nxt);
-    compute(1, cur, cur_fl);
-    FA_TRACE_ONLY(++tr_tiles;)
-    cur = nxt; cur_fl = it.flags;
-  }
+  // the tile stream; one loop per form (halved tiles or not), so that neither pays for the other's registers
+  auto stream = [&](auto nb_c) __attribute__((always_inline)) {
+    while (cur >= 0) {
+      int nxt = it.next(dec);
+      wait_async_loads();
+      __syncthreads();
+      if (nxt >= 0) issue(1, nxt);
+      compute(0, cur, cur_fl, nb_c);
+      FA_TRACE_ONLY(++tr_tiles;)
+      cur = nxt; cur_fl = it.flags;
+      if (cur < 0) break;
+      nxt = it.next(dec);
+      wait_async_loads();
+      __syncthreads();
+      if (nxt >= 0) issue(0, nxt);
+      compute(1, cur, cur_fl, nb_c);
+      FA_TRACE_ONLY(++tr_tiles;)
+      cur = nxt; cur_fl = it.flags;
+    }
+  };
+  if (halved) stream(IntC<1>{}); else stream(IntC<2>{});
   FA_STAMP(g_trace_fwd, 3, FA_CLOCK()); FA_STAMP(g_trace_fwd, 5, tr_tiles);
 
+  if (halved) {
+    // The wave that took the second half of every key tile hands its softmax state (reference point, partial
+    // row sum, unnormalised O) to the wave that took the first half of the same rows, lane for lane, through
+    // the LDS the tile stream no longer needs; that wave merges the two and goes on alone.
+    constexpr int NV = 2 + 16 * DBN;
+    __syncthreads();   // every wave is done with the last tile
+    float* mb = reinterpret_cast<float*>(smem) + qc.rb * (NV * 64) + lane;
+    if (sub == 1) {
+      mb[0] = m_ref; mb[64] = l_run;
+#pragma unroll
+      for (int db = 0; db < DBN; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mb[(2 + 16 * db + r) * 64] = o[db][r];
+    }
+    __syncthreads();
+    if (sub == 0) {
+      const float m_b = mb[0], l_b = mb[64];
+      const float m_new = fmaxf(m_ref, m_b);
+      const float ca = fast_exp2(m_ref - m_new), cb = fast_exp2(m_b - m_new);   // both unset: 1 and 1 on zeros
+      m_ref = m_new;
+      l_run = l_run * ca + l_b * cb;
+#pragma unroll
+      for (int db = 0; db < DBN; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] = o[db][r] * ca + mb[(2 + 16 * db + r) * 64] * cb;
+    }
+  }
+  const bool writer = !halved || sub == 0;   // the wave that holds the rows' result
   const float l_tot = xhalf_sum(l_run);
   if (DOC && nsplit > 1) {
     // This workgroup saw one chunk of the keys: store the unnormalised partial result; the last
@@ -295,13 +369,13 @@ void fwd_kernel(const KArgs a) {
     const int64_t tbase = (int64_t(b) * a.H + h) * a.split_tiles + wk.gt;
     float* po = a.sk_o + (tbase * a.split_k + wk.split) * (128 * D);
     float* pml = a.sk_ml + (tbase * a.split_k + wk.split) * (128 * 2);
-    const int rt = (threadIdx.x >> 6) * 32 + (lane & 31);   // row inside the tile
-    if (g == 0) store_dev(pml + rt * 2, m_ref, l_tot);
+    const int rt = qc.rb * 32 + (lane & 31);   // row inside the tile
+    if (g == 0 && writer) store_dev(pml + rt * 2, m_ref, l_tot);
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        if (32 * db + 8 * q4 >= D) continue;
+        if (32 * db + 8 * q4 >= D || !writer) continue;
         f32x4 x = {o[db][4 * q4 + 0], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]};
         store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
       }
@@ -392,7 +466,7 @@ void fwd_kernel(const KArgs a) {
 
   // epilogue: normalise, write O and LSE
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  if (row >= 0) {
+  if (row >= 0 && writer) {
     if (g == 0) lsep[row] = l_tot > 0.f ? m_ref + fast_log2(l_tot) : -INFINITY;
     T* orow = op + int64_t(row) * a.o_rs;
 #pragma unroll

@@ -273,6 +273,12 @@ struct QTileCtx {
   int low_i;                               // first key this lane's row may see (sliding window; very negative: none)
   int w_lowmin, w_lowmax;                  // smallest / largest such bound among the wave's rows
   bool glob_i;                             // this lane's row has an id >= 0 (sees every id)
+  // A tile with at most 64 rows (the last tile of the global rows, a short query block) would leave two of
+  // the four waves without rows.  Then waves 2, 3 take the rows of waves 0, 1 as well (rb = row block of the
+  // wave) and the pair splits every key tile between them: wave `sub` computes the 32-key half `sub` with a
+  // softmax state (or dQ sum) of its own, and the two are merged once, after the tile loop.
+  int rb, sub;
+  bool halved;
   const int* ekp;
   const IdSummary* ksum;
 
@@ -287,8 +293,11 @@ struct QTileCtx {
     g_kfirst = 0; g_klast = 0x3fffffff;
     gp = DOC ? 0 : a.gap;
     int posc;   // r of this lane's row, 0 if none
+    rb = wave; sub = 0; halved = false;
     if (!DOC) {
-      const int m0 = tile * 128, mw = m0 + wave * 32;
+      const int m0 = tile * 128;
+      if (a.M - m0 <= 64 && a.bmask == nullptr) { halved = true; rb = wave & 1; sub = wave >> 1; }
+      const int mw = m0 + rb * 32;
       row = mw + lq < a.M ? mw + lq : -1;
       w_rmin = mw; w_rmax = min(mw + 31, a.M - 1);
       if (w_rmax < w_rmin) w_rmax = -1;
@@ -299,7 +308,9 @@ struct QTileCtx {
       ksum = a.ksum + b * a.ks_bs + h * a.ks_hs;
       const IdSummary* qs = a.qsum + b * a.qs_bs + h * a.qs_hs + 2 * tile;
       const IdSummary s0 = qs[0], s1 = qs[1];
-      const int64_t pos = b * a.pm_bs + h * a.pm_hs + tile * 128 + wave * 32 + lq;
+      // (the rows of a tile sit at its front: padding only follows the last local and the last global row)
+      if (s0.nvalid + s1.nvalid <= 64) { halved = true; rb = wave & 1; sub = wave >> 1; }
+      const int64_t pos = b * a.pm_bs + h * a.pm_hs + tile * 128 + rb * 32 + lq;
       row = a.perm[pos];     // issued together with the summaries: no dependent load chain
       eq_i = a.peq[pos];
       const int ps = a.ppos[pos];
@@ -510,6 +521,24 @@ FA_DEV bool split_arrive(int* counter, int nsplit) {
   return sk_last != 0;
 }
 
+// Which leading keys of (batch b, key head hk) the column kernel of dk/dv takes (see kGcolTilesMax): `ncols`
+// keys, a multiple of 128 (0: none), seen by `tiles` 64-row tiles of global rows in all.  Both kernels of a
+// launch evaluate this, so the key range is cut in the same place.
+struct GcolInfo { int ncols, tiles; };
+FA_DEV GcolInfo gcol_info(const KArgs& a, int b, int hk) {
+  int k0 = 0x7fffffff, tiles = 0;
+  for (int gi = 0; gi < a.G; ++gi) {
+    const QHeader hd = a.qhdr[b * a.qh_bs + (hk * a.G + gi) * a.qh_hs];
+    k0 = min(k0, hd.k0);
+    tiles += (hd.nG + 63) / 64;
+  }
+  GcolInfo r;
+  r.tiles = tiles;
+  r.ncols = k0 >= a.nKs ? (a.N + 127) / 128 * 128 : (k0 * kSumRows) / 128 * 128;
+  if (tiles > kGcolTilesMax) r.ncols = 0;
+  return r;
+}
+
 // blockIdx -> (tile, batch*head) for grids of `ntile` tiles per (batch, head); grid_blocks() is the
 // matching grid size.  Consecutive workgroup ids land on different XCDs (8 of them, each with its
 // own L2), so the map decides which XCD's L2 sees which head:
@@ -531,8 +560,9 @@ FA_HD int grid_blocks(int ntile, int BH) {
   return (BH * ntile + 7) / 8 * 8;
 }
 
-FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, int& bh) {
-  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+// bid: index of the workgroup (blockIdx.x, unless several forms share one grid).
+FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, int& bh, int bid) {
+  const int xcd = bid & 7, idx = bid >> 3;
   if (BH % 8 == 0) {
     const int heads = BH / 8;  // heads per XCD
     if (tile_major) {
@@ -550,9 +580,12 @@ FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, in
     tile_slot = idx * k + xcd % k;
     return tile_slot < ntile;
   }
-  tile_slot = int(blockIdx.x) / BH;
-  bh = int(blockIdx.x) % BH;
+  tile_slot = bid / BH;
+  bh = bid % BH;
   return tile_slot < ntile;
+}
+FA_DEV bool block_to_tile(int ntile, int BH, bool tile_major, int& tile_slot, int& bh) {
+  return block_to_tile(ntile, BH, tile_major, tile_slot, bh, (int)blockIdx.x);
 }
 
 }  // namespace fa
