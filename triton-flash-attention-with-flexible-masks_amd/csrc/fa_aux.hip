@@ -31,13 +31,12 @@ FA_DEV int wave_max(int v) {
 
 // Key side: one wave per summary tile of 64 keys; 4 tiles per workgroup.
 template <bool I64>
-__global__ __launch_bounds__(256) void plan_k_kernel(const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
-                                                     int L, int Lp, int nS, int H1, int* __restrict__ out32,
-                                                     IdSummary* __restrict__ sum) {
+FA_DEV void plan_k_body(const int bx, const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
+                        int L, int Lp, int nS, int H1, int* __restrict__ out32, IdSummary* __restrict__ sum) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int tile = blockIdx.x * 4 + wave;
-  if (tile >= nS) return;
+  const int tile = bx * 4 + wave;
   const int h = blockIdx.y, b = blockIdx.z;
+  if (tile >= nS || h >= H1) return;
   const int r = tile * kSumRows + lane;
   const bool valid = r < L;
   const int v = valid ? load_id<I64>(ids, b * s_b + h * s_h + int64_t(r) * s_r) : 0;
@@ -58,13 +57,14 @@ __global__ __launch_bounds__(256) void plan_k_kernel(const void* __restrict__ id
 constexpr int kPlanChunk = 1024;
 
 template <bool I64>
-__global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
-                                                         int M, int Mp, int Pp, int nCh, int H1, int* __restrict__ eq32,
-                                                         int* __restrict__ perm, int* __restrict__ peq,
-                                                         int* __restrict__ ppos, int* __restrict__ cnt) {
+FA_DEV void plan_count_body(const int ch, const void* __restrict__ ids, int64_t s_b, int64_t s_h, int64_t s_r,
+                            int M, int Mp, int Pp, int nCh, int H1, int* __restrict__ eq32,
+                            int* __restrict__ perm, int* __restrict__ peq,
+                            int* __restrict__ ppos, int* __restrict__ cnt) {
   __shared__ int sh[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.y, b = blockIdx.z;
+  if (h >= H1) return;   // (uniform over the workgroup)
   const int64_t bh = int64_t(b) * H1 + h;
   const int64_t base = b * s_b + h * s_h;
   int c = 0;
@@ -89,6 +89,18 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const void* __restrict_
   if (lane == 0) sh[wave] = c;
   __syncthreads();
   if (tid == 0) cnt[bh * nCh + ch] = sh[0] + sh[1] + sh[2] + sh[3];
+}
+
+// The two kernels above in one launch (they do not depend on each other, and every launch of a kernel this
+// small costs more in the gap to the next one than in its run time): workgroups [0, nKb) take the key side,
+// the rest the query side; grid.y covers the larger of the two head counts.
+struct PlanSide { const void* ids; int64_t s_b, s_h, s_r; int L, Lp, H1; };
+template <bool I64>
+__global__ __launch_bounds__(256) void plan_kc_kernel(PlanSide k, int nS, int nKb, int* __restrict__ ek32, IdSummary* __restrict__ ksum,
+                                                      PlanSide q, int Pp, int nCh, int* __restrict__ eq32, int* __restrict__ perm,
+                                                      int* __restrict__ peq, int* __restrict__ ppos, int* __restrict__ cnt) {
+  if ((int)blockIdx.x < nKb) plan_k_body<I64>(blockIdx.x, k.ids, k.s_b, k.s_h, k.s_r, k.L, k.Lp, nS, k.H1, ek32, ksum);
+  else plan_count_body<I64>(blockIdx.x - nKb, q.ids, q.s_b, q.s_h, q.s_r, q.L, q.Lp, Pp, nCh, q.H1, eq32, perm, peq, ppos, cnt);
 }
 
 // Step 2: stable two-way partition.  Every chunk derives its output offsets from the counts of
@@ -220,22 +232,18 @@ int launch_mask_plan(const fa_params* p, const WsLayout& w, hipStream_t s) {
   IdSummary* ksum = reinterpret_cast<IdSummary*>(ws + w.off_ksum);
   hipError_t e;
   {
-    const int64_t* st = p->ek_stride;
-    dim3 grid((w.nKs + 3) / 4, w.Hk1, p->B);
+    const int64_t* sk = p->ek_stride;
+    const int64_t* sq = p->eq_stride;
+    const PlanSide ks = {p->ek, sk[0], sk[1], sk[2], p->N, w.Np, w.Hk1};
+    const PlanSide qs = {p->eq, sq[0], sq[1], sq[2], p->M, w.Mp, w.Hq1};
+    const int nKb = (w.nKs + 3) / 4;
+    dim3 grid_kc(nKb + w.nCh, w.Hk1 > w.Hq1 ? w.Hk1 : w.Hq1, p->B);
     if (i64)
-      hipLaunchKernelGGL(plan_k_kernel<true>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, ek32, ksum);
+      hipLaunchKernelGGL(plan_kc_kernel<true>, grid_kc, dim3(256), 0, s, ks, w.nKs, nKb, ek32, ksum, qs, w.Pp, w.nCh, eq32, perm, peq, ppos, cnt);
     else
-      hipLaunchKernelGGL(plan_k_kernel<false>, grid, dim3(256), 0, s, p->ek, st[0], st[1], st[2], p->N, w.Np, w.nKs, w.Hk1, ek32, ksum);
+      hipLaunchKernelGGL(plan_kc_kernel<false>, grid_kc, dim3(256), 0, s, ks, w.nKs, nKb, ek32, ksum, qs, w.Pp, w.nCh, eq32, perm, peq, ppos, cnt);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
-  }
-  {
-    const int64_t* st = p->eq_stride;
     dim3 grid(w.nCh, w.Hq1, p->B);
-    if (i64)
-      hipLaunchKernelGGL(plan_count_kernel<true>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, ppos, cnt);
-    else
-      hipLaunchKernelGGL(plan_count_kernel<false>, grid, dim3(256), 0, s, p->eq, st[0], st[1], st[2], p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, perm, peq, ppos, cnt);
-    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     const int gap = p->N > p->M ? p->N - p->M : 0;
     hipLaunchKernelGGL(plan_scatter_kernel, grid, dim3(256), 0, s, p->M, w.Mp, w.Pp, w.nCh, w.Hq1, eq32, cnt, perm, peq, ppos,
                        p->causal ? p->qpos : nullptr, p->qpos_stride, gap, hdr);
