@@ -304,6 +304,7 @@ void bwd_dq_kernel(const KArgs a) {
         for (int u = 0; u < IT; ++u) {
           const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
           mrow[u] = i < 128 * C4 ? prm[r] : -1;
+          if (mrow[u] < 0) continue;   // no such row: nothing to fetch
 #pragma unroll
           for (int sp = 0; sp < NS; ++sp) x[u][sp] = load_dev4(bo + min(sp, nsplit - 1) * (128 * D) + r * D + 4 * c);
         }

@@ -407,6 +407,7 @@ void fwd_kernel(const KArgs a) {
         for (int u = 0; u < IT; ++u) {
           const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
           mrow[u] = i < 128 * C4 ? prm[r] : -1;
+          if (mrow[u] < 0) continue;   // no such row (a tile of a few dozen rows has mostly these): nothing to fetch
 #pragma unroll
           for (int sp = 0; sp < NS; ++sp) {
             const int spc = min(sp, nsplit - 1);   // chunks past the last one repeat it (weight 0 below)
