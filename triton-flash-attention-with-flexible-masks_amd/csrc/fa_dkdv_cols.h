@@ -267,7 +267,7 @@ FA_DEV void dkdv_cols_body(const KArgs& a, const int bid, char* smem) {
         const char* tr = smem + r * 2 * TILE_BYTES + (which == 0 ? TILE_BYTES : 0);   // dO^T for dV, Q^T for dK
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-          constexpr int NM = 2 * DBN, PRE = NM < 3 ? NM : 3;
+          constexpr int NM = 2 * DBN, PRE = NM < 2 ? NM : 2;
           int t0 = tr0[0], t1 = tr0[1];
           asm volatile("" : "+v"(t0), "+v"(t1));
           auto tr_off = [&](const int db, const int hh) __attribute__((always_inline)) { return (hh ? t1 : t0) ^ (db << 6); };

@@ -319,7 +319,7 @@ void fwd_kernel(const KArgs a) {
       __syncthreads();
       if (nxt >= 0) issue(1, nxt);
       compute(0, cur, cur_fl, nb_c);
-      FA_TRACE_ONLY(++tr_tiles;)
+      FA_TRACE_ONLY(tr_tiles = __builtin_amdgcn_readfirstlane(tr_tiles + 1);)   // (kept scalar: as a plain counter it cost 19 spilled registers)
       cur = nxt; cur_fl = it.flags;
       if (cur < 0) break;
       nxt = it.next(dec);
@@ -327,7 +327,7 @@ void fwd_kernel(const KArgs a) {
       __syncthreads();
       if (nxt >= 0) issue(0, nxt);
       compute(1, cur, cur_fl, nb_c);
-      FA_TRACE_ONLY(++tr_tiles;)
+      FA_TRACE_ONLY(tr_tiles = __builtin_amdgcn_readfirstlane(tr_tiles + 1);)   // (kept scalar: as a plain counter it cost 19 spilled registers)
       cur = nxt; cur_fl = it.flags;
     }
   };
