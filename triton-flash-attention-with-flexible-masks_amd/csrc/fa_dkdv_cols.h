@@ -247,11 +247,7 @@ FA_DEV void dkdv_cols_body(const KArgs& a, const int bid, char* smem) {
       }
     }
     // the next 32 keys of this wave: K and V rows travel while this block's second products run
-#ifdef FA_EXP_NOLOAD
-    const bool more = false;
-#else
     const bool more = j + NW < nblk && nres > 0;
-#endif
     __builtin_amdgcn_sched_barrier(0);
     if (more) load_kv(j + NW);
     __builtin_amdgcn_sched_barrier(0);
@@ -312,20 +308,16 @@ FA_DEV void dkdv_cols_body(const KArgs& a, const int bid, char* smem) {
                 *reinterpret_cast<typename E::vec4*>(xp + (lq & 15) * kXpPitch + (32 * dd + 8 * q4 + 4 * g) * 2) = xk;
               }
           }
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          asm volatile("" ::: "memory");   // (order only: the LDS executes a wave's operations in issue order)
 #pragma unroll
           for (int i = 0; i < XP_NI; ++i) {
             const int kr = XP_RPI * i + lane / XP_CPR, cc = lane % XP_CPR;   // key row of the half block, 16-byte chunk of its row
             const vec8 x = *reinterpret_cast<const vec8*>(xp + kr * kXpPitch + cc * 16);
             const int key_o = nw + 16 * kh + kr;
-#ifndef FA_EXP_NOSTORE
             if (key_o < a.N && 32 * d0 + 8 * cc < D)
-#else
-            if (key_o < -5)
-#endif
               *reinterpret_cast<vec8*>(reinterpret_cast<char*>(obase) + ((unsigned)key_o * ors_b + (unsigned)(64 * d0 + 16 * cc))) = x;
           }
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads are done before the patch is overwritten
+          asm volatile("" ::: "memory");   // the next writes to the patch are issued, hence executed, after these reads
         }
       }
     };
