@@ -1084,7 +1084,14 @@ def test_case_found_outside_the_bound(case):
     (oracle.attention_grads(store_dtype=...), output rounded too) reaches 0.92 of the bound on the same inputs
     at another element; the kernel's O differs from the model's by one bf16 step in places (other summation
     order), which makes its delta another draw from the same error distribution: here the kernel is less
-    accurate than an implementation that rounds exactly where the reference rounds.
+    accurate than an implementation that rounds exactly where the reference rounds.  Recomputed on the CPU with
+    the kernel's own O, the excess comes from one element of dS: magnitude 10 (dP - delta = 27.8, P = 0.359),
+    1.5e-4 away from a bf16 rounding tie (9.9686 between 9.9375 and 10.0).  Its half-step error of 0.031 is worth
+    0.0083 in dK, 40 % of the bound, whichever way it falls: with the exact P it falls down and cancels the delta
+    error of the other 135 rows of that column, with P rounded to the 11 bits of the fp16 hand-over between the
+    wave pair (or to 8) it falls up and adds to it.  The hand-over is the one place where this kernel rounds and the
+    reference does not (flash_triton.py:301 keeps P in fp32), but it acts as the tie-breaker of a rounding of dS
+    that the reference performs too (flash_triton.py:306).
     Second and third case (5 and 4 keys in all, 180 and 215 query rows with per-row positions, 1.0-1.6 kept keys
     per row, 55 rows per key): 1.09 of the bound -- and the CPU model of the reference's roundings is itself at
     1.06 and 1.09 of it there: no implementation that rounds where the reference rounds meets the bound on
