@@ -44,6 +44,7 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "triton-flash-attention-with-flexible-masks_amd"))
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}   # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0   # MI355X HBM3E
 HBM_PEAK_GBS = 8000.0
 
 KERNEL_OF = {"fa_fwd": "fwd_kernel", "fa_bwd_dq": "bwd_dq_kernel", "fa_bwd_dkdv": "bwd_dkdv_kernel"}
@@ -279,6 +280,15 @@ def measure_other_config(name, torch, steps=20, warmup=5):
     if ex is not None:
         out["tflops_executed"] = round((ex["fwd"] + ex["dq"] + ex["dkdv"]) / ms * 1e-9, 1)
         out["pct_of_mfma_peak"] = round(100 * out["tflops_executed"] / PEAK_TFLOPS[w.dtype], 2)
+    # The other roof: the bytes a step cannot avoid (every operand and result of the three kernels once:
+    # forward Q K V -> O; dq Q K V dO O -> dQ; dk/dv Q dO K V -> dK dV) over the 8 TB/s HBM peak.  For a
+    # configuration whose few global rows make every head stream all of K and V (cfg5) this, not the MFMA
+    # share, says how far the step is from its bound.
+    es = 4 if w.dtype == "fp32" else 2
+    nq, nk = w.B * w.H * w.Lq * w.D * es, w.B * w.Hk * w.Lk * w.D * es
+    gb = ((2 * nq + 2 * nk) + (4 * nq + 2 * nk) + (2 * nq + 4 * nk)) * 1e-9
+    out["hbm_gb_min"] = round(gb, 3)
+    out["pct_of_hbm_peak"] = round(100 * gb / (ms * 1e-3) / (PEAK_HBM_GBS), 2)
     return out
 
 
