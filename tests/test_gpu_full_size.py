@@ -222,3 +222,60 @@ def test_packed_prefill_with_per_sequence_alignment_at_16k_keys():
         assert (sq(out.detach().float().cpu()) - ro).abs().max().item() <= TOL_O
         for nm, got, ref, sl in (("dq", qd.grad, rdq, sq), ("dk", kd.grad, rdk, sk), ("dv", vd.grad, rdv, sk)):
             check_close(f"sequence {s} {nm}", sl(got.float().cpu()), ref)
+
+
+def test_tensors_larger_than_4_gib():
+    """Every tensor of the call larger than 4 GiB (B=34, H=32, L=16384, D=128, bf16: 4.56 GB each; causal + the
+    headline configuration's ids): an index that was formed in 32 bits somewhere would land in the wrong
+    (batch, head).  Every head through the size-independent properties, with and without ids, evaluated on the GPU (V = 1 and
+    dO = 1: O is one on every row, the column sums of dV add up to the number of rows), and four slices --
+    the first, one whose offset lies past 2^31 bytes, one past 2^31 elements and the very last -- against the oracle."""
+    from flash_mi355 import attention, attention_with_lse, workloads as W, SCORE_FUNC_MODE1_DOC
+    from oracle import attention_oracle as O
+    w = W.make_workload("cfg4_doc_causal_16k")
+    B, H, L, D = 34, 32, w.Lq, w.D
+    assert B * H * L * D * 2 > 2 ** 32 and (L, D) == (16384, 128)
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * 2 ** 30:
+        pytest.skip("needs 60 GB of free device memory")
+    dev = torch.device("cuda")
+    print(f"case tensors of {B * H * L * D * 2 / 2 ** 30:.2f} GiB", flush=True)
+    ids = torch.from_numpy(w.eq[0]).to(dev)[None, None, :].expand(B, H, L)
+    g = torch.Generator(device=dev).manual_seed(11)
+    q = torch.randn(B, H, L, D, device=dev, dtype=torch.bfloat16, generator=g)
+    k = torch.randn(B, H, L, D, device=dev, dtype=torch.bfloat16, generator=g)
+
+    ones_v = torch.ones(B, H, L, D, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    out = attention(q, k, ones_v, True, None, ids, ids, SCORE_FUNC_MODE1_DOC)
+    assert (out.detach().float() - 1.0).abs().amax().item() <= 2 ** -7   # causal with ids: every row sees itself
+    out.backward(torch.ones_like(out))
+    col = ones_v.grad.float().sum(dim=2)                               # [B, H, D]
+    assert ((col - L).abs() / L).amax().item() <= 5e-3
+    # the same without ids (the dense forms of the three kernels)
+    ones_v.grad = None
+    out = attention(q, k, ones_v, True, None)
+    assert (out.detach().float() - 1.0).abs().amax().item() <= 2 ** -7
+    out.backward(torch.ones_like(out))
+    col = ones_v.grad.float().sum(dim=2)
+    assert ((col - L).abs() / L).amax().item() <= 5e-3
+    del out, col, ones_v
+    torch.cuda.empty_cache()
+
+    v = torch.randn(B, H, L, D, device=dev, dtype=torch.bfloat16, generator=g)
+    do = torch.randn(B, H, L, D, device=dev, dtype=torch.bfloat16, generator=g)
+    qd, kd, vd = (t.requires_grad_(True) for t in (q, k, v))
+    out, lse = attention_with_lse(qd, kd, vd, True, None, ids, ids, SCORE_FUNC_MODE1_DOC)
+    out.backward(do)
+    torch.cuda.synchronize()
+    eq1 = torch.from_numpy(w.eq[0])[None, None, :]
+    assert (16 * H + 13) * L * D * 2 > 2 ** 31 and (32 * H + 5) * L * D > 2 ** 31
+    for (b, h) in ((0, 0), (16, 13), (32, 5), (B - 1, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        print(f"  slice ({b},{h})", flush=True)
+        ro, rl, rdq, rdk, rdv = O.attention_autograd(q[sl].detach().cpu(), k[sl].detach().cpu(), v[sl].detach().cpu(), do[sl].cpu(),
+                                                      True, None, eq1, eq1, 1)
+        assert not torch.isinf(rl).any()
+        assert (lse[sl].detach().cpu() - rl).abs().max().item() <= TOL_LSE
+        assert (out[sl].detach().float().cpu() - ro).abs().max().item() <= TOL_O
+        for nm, got, ref in (("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+            check_close(f"4 GiB tensors, slice ({b},{h}) {nm}", got[sl].cpu(), ref)
