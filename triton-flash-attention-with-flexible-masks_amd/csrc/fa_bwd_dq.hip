@@ -272,14 +272,13 @@ void bwd_dq_kernel(const KArgs a) {
     // adds them up in a fixed order and writes dQ.
     const int64_t tbase = (int64_t(b) * a.H + h) * a.split_tiles + wk.gt;
     float* po = a.sk_o + (tbase * a.split_k + wk.split) * (128 * D);
-    const int rt = qc.rb * 32 + (lane & 31);   // row inside the tile
 #pragma unroll
     for (int db = 0; db < DBN; ++db)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         if (32 * db + 8 * q4 >= D || !writer) continue;
         f32x4 x = {dq[db][4 * q4 + 0], dq[db][4 * q4 + 1], dq[db][4 * q4 + 2], dq[db][4 * q4 + 3]};
-        store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
+        store_dev(po + part_index<D>(qc.rb, 4 * db + q4, lane) * 4, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_dq, 4, FA_CLOCK()); return; }
     FA_STAMP(g_trace_dq, 6, FA_CLOCK());
@@ -299,14 +298,17 @@ void bwd_dq_kernel(const KArgs a) {
       constexpr int IT = decltype(it_c)::value, NS = decltype(ns_c)::value;
       for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
         f32x4 x[IT][NS];
-        int mrow[IT];
+        int mrow[IT], cc[IT];
 #pragma unroll
         for (int u = 0; u < IT; ++u) {
-          const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
+          const int i = i0 + 256 * u;
+          int r, c;
+          part_coords<D>(min(i, 128 * C4 - 1), r, c);
+          cc[u] = c;
           mrow[u] = i < 128 * C4 ? prm[r] : -1;
           if (mrow[u] < 0) continue;   // no such row: nothing to fetch
 #pragma unroll
-          for (int sp = 0; sp < NS; ++sp) x[u][sp] = load_dev4(bo + min(sp, nsplit - 1) * (128 * D) + r * D + 4 * c);
+          for (int sp = 0; sp < NS; ++sp) x[u][sp] = load_dev4(bo + min(sp, nsplit - 1) * (128 * D) + i * 4);
         }
 #pragma unroll
         for (int u = 0; u < IT; ++u) {
@@ -317,7 +319,7 @@ void bwd_dq_kernel(const KArgs a) {
             const float w = sp < nsplit ? 1.f : 0.f;
             acc[0] += w * x[u][sp][0]; acc[1] += w * x[u][sp][1]; acc[2] += w * x[u][sp][2]; acc[3] += w * x[u][sp][3];
           }
-          finish_row(mrow[u], (i0 + 256 * u) % C4, acc);
+          finish_row(mrow[u], cc[u], acc);
         }
       }
     };
@@ -328,12 +330,13 @@ void bwd_dq_kernel(const KArgs a) {
       return;
     }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
-      const int r = i / C4, c = i % C4;
+      int r, c;
+      part_coords<D>(i, r, c);
       const int mrow = prm[r];
       if (mrow < 0) continue;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
       for (int sp = 0; sp < nsplit; ++sp) {
-        const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
+        const f32x4 x = load_dev4(bo + sp * (128 * D) + i * 4);
         acc[0] += x[0]; acc[1] += x[1]; acc[2] += x[2]; acc[3] += x[3];
       }
       finish_row(mrow, c, acc);

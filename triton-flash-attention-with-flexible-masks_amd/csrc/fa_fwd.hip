@@ -377,7 +377,7 @@ void fwd_kernel(const KArgs a) {
       for (int q4 = 0; q4 < 4; ++q4) {
         if (32 * db + 8 * q4 >= D || !writer) continue;
         f32x4 x = {o[db][4 * q4 + 0], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]};
-        store_dev(po + rt * D + 32 * db + 8 * q4 + 4 * g, x);
+        store_dev(po + part_index<D>(qc.rb, 4 * db + q4, lane) * 4, x);
       }
     if (!split_arrive(a.sk_cnt + tbase, nsplit)) { FA_STAMP(g_trace_fwd, 4, FA_CLOCK()); return; }
     FA_STAMP(g_trace_fwd, 6, FA_CLOCK());
@@ -402,17 +402,20 @@ void fwd_kernel(const KArgs a) {
       for (int i0 = threadIdx.x; i0 < 128 * C4; i0 += 256 * IT) {
         float m_[IT][NS], l_[IT][NS];
         f32x4 x[IT][NS];
-        int mrow[IT];
+        int mrow[IT], cc[IT];
 #pragma unroll
         for (int u = 0; u < IT; ++u) {
-          const int i = i0 + 256 * u, r = min(i / C4, 127), c = i % C4;
+          const int i = i0 + 256 * u;
+          int r, c;
+          part_coords<D>(min(i, 128 * C4 - 1), r, c);
+          cc[u] = c;
           mrow[u] = i < 128 * C4 ? prm[r] : -1;
           if (mrow[u] < 0) continue;   // no such row (a tile of a few dozen rows has mostly these): nothing to fetch
 #pragma unroll
           for (int sp = 0; sp < NS; ++sp) {
             const int spc = min(sp, nsplit - 1);   // chunks past the last one repeat it (weight 0 below)
             load_dev(bml + spc * 256 + r * 2, m_[u][sp], l_[u][sp]);
-            x[u][sp] = load_dev4(bo + spc * (128 * D) + r * D + 4 * c);
+            x[u][sp] = load_dev4(bo + spc * (128 * D) + i * 4);
           }
         }
 #pragma unroll
@@ -429,7 +432,7 @@ void fwd_kernel(const KArgs a) {
             lsum += w * l_[u][sp];
             acc[0] += w * x[u][sp][0]; acc[1] += w * x[u][sp][1]; acc[2] += w * x[u][sp][2]; acc[3] += w * x[u][sp][3];
           }
-          finish_row(mrow[u], (i0 + 256 * u) % C4, mmax, lsum, acc);
+          finish_row(mrow[u], cc[u], mmax, lsum, acc);
         }
       }
     };
@@ -440,7 +443,8 @@ void fwd_kernel(const KArgs a) {
       return;
     }
     for (int i = threadIdx.x; i < 128 * C4; i += 256) {
-      const int r = i / C4, c = i % C4;
+      int r, c;
+      part_coords<D>(i, r, c);
       const int mrow = prm[r];
       if (mrow < 0) continue;
       float mmax = -INFINITY;
@@ -456,7 +460,7 @@ void fwd_kernel(const KArgs a) {
         load_dev(bml + sp * 256 + r * 2, m_, l_);
         const float w = m_ == -INFINITY ? 0.f : fast_exp2(m_ - mmax);
         lsum += w * l_;
-        const f32x4 x = load_dev4(bo + sp * (128 * D) + r * D + 4 * c);
+        const f32x4 x = load_dev4(bo + sp * (128 * D) + i * 4);
         acc[0] += w * x[0]; acc[1] += w * x[1]; acc[2] += w * x[2]; acc[3] += w * x[3];
       }
       finish_row(mrow, c, mmax, lsum, acc);

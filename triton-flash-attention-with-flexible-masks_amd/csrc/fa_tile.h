@@ -484,11 +484,26 @@ FA_DEV void store_dev(float* p, float x0, float x1) {
   const u64 v = (u64)__float_as_uint(x0) | ((u64)__float_as_uint(x1) << 32);
   __hip_atomic_store(reinterpret_cast<u64*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16 bytes with the same cache policy as the 8-byte device-scope store above (the `sc1` bit); not atomic as
+// a whole, which the partial results do not need: they are read after the arrival counter says so.
+// The wait states behind it are part of the instruction as far as this code is concerned: a vector instruction that
+// writes the data registers of a store wider than 8 bytes must not follow it directly, and the compiler, which
+// keeps that distance for its own stores, does not look inside inline assembly (it placed an address computation
+// into the first data register right behind the store).
 FA_DEV void store_dev(float* p, f32x4 x) {
-  // elements go through scalars: a bit cast applied to a vector element reads element 0
-  const float x0 = x[0], x1 = x[1], x2 = x[2], x3 = x[3];
-  store_dev(p, x0, x1);
-  store_dev(p + 2, x2, x3);
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" :: "v"(p), "v"(x) : "memory");
+}
+// A partial [128 rows x D] fp32 tile lies in the scratch in the accumulator order of the waves that own the
+// rows, not row by row: float4 number i = (rb * (D / 8) + grp) * 64 + lane holds the columns 8 * grp +
+// 4 * (lane >> 5) .. + 3 of row 32 * rb + (lane & 31).  A wave's store instruction then writes 1 KB in one
+// piece (row by row it was 64 pieces of 16 bytes), and the merging workgroup reads float4 i with thread i.
+template <int D>
+FA_DEV int part_index(int rb, int grp, int lane) { return (rb * (D / 8) + grp) * 64 + lane; }
+template <int D>
+FA_DEV void part_coords(int i, int& r, int& c) {   // row of the tile and float4 of that row
+  const int rbq = i >> 6, lane = i & 63, rb = rbq / (D / 8), grp = rbq % (D / 8);
+  r = rb * 32 + (lane & 31);
+  c = 2 * grp + (lane >> 5);
 }
 FA_DEV void load_dev(const float* p, float& x0, float& x1) {
   typedef unsigned long long u64;
