@@ -638,20 +638,16 @@ void bwd_dkdv_kernel(const KArgs a) {
   FA_STAMP(g_trace_dkdv, 4, FA_CLOCK()); FA_STAMP(g_trace_dkdv, 6, tr_tiles);
   // shader clocks the first gradient wave spent at the pair flag (role-split form)
   FA_TRACE_ONLY(if (SPLIT && threadIdx.x == 64 * NKB && blockIdx.x < fa::kTraceWgs) g_trace_dkdv[blockIdx.x * 8 + 1] = tr_wait;)
-  if (key < a.N) {
-    T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs + int64_t(key) * a.dv_rs;
-    T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs + int64_t(key) * a.dk_rs;
-    auto store = [&](T* orow, const f32x16 (&v)[DBN], const float sc) __attribute__((always_inline)) {
-#pragma unroll
-      for (int db = 0; db < DBN; ++db)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
-          const typename E::vec2 k0 = E::cvt2(v[db][4 * q4 + 0] * sc, v[db][4 * q4 + 1] * sc);
-          const typename E::vec2 k1 = E::cvt2(v[db][4 * q4 + 2] * sc, v[db][4 * q4 + 3] * sc);
-          typename E::vec4 xk = {k0[0], k0[1], k1[0], k1[1]};
-          *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = xk;
-        }
+  {
+    // dK / dV rows leave through LDS (store_rows_through_lds), once every wave is done with the last query tile
+    T* dvp = reinterpret_cast<T*>(a.dv) + b * a.dv_bs + hk * a.dv_hs;
+    T* dkp = reinterpret_cast<T*>(a.dk) + b * a.dk_bs + hk * a.dk_hs;
+    __syncthreads();
+    char* patch = smem + wave * row_patch_bytes<D>();
+    auto store = [&](T* base, const int64_t rs, const f32x16 (&v)[DBN], const float sc) __attribute__((always_inline)) {
+      store_rows_through_lds<E, D, DBN>(patch, v, sc, [&](const int r) -> T* {
+        return nw + r < a.N ? base + int64_t(nw + r) * rs : nullptr;
+      });
     };
     if (SPLIT) {
       if (role == 1 && pair_lost) {   // the bounded wait expired somewhere: this wave's dK is not to be trusted
@@ -661,10 +657,10 @@ void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[db][r] = __builtin_nanf("");
       }
-      store(role == 0 ? dvrow : dkrow, acc, role == 0 ? 1.0f : a.scale);
+      if (role == 0) store(dvp, a.dv_rs, acc, 1.0f); else store(dkp, a.dk_rs, acc, a.scale);
     } else {
-      store(dvrow, acc, 1.0f);
-      store(dkrow, acc2, a.scale);
+      store(dvp, a.dv_rs, acc, 1.0f);
+      store(dkp, a.dk_rs, acc2, a.scale);
     }
   }
   }   // run of key tiles

@@ -345,19 +345,15 @@ void bwd_dq_kernel(const KArgs a) {
     return;
   }
 
-  if (row >= 0 && writer) {
-    T* drow = dqp + int64_t(row) * a.dq_rs;
-    const float sc = a.scale;
-#pragma unroll
-    for (int db = 0; db < DBN; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
-        const typename E::vec2 x0 = E::cvt2(dq[db][4 * q4 + 0] * sc, dq[db][4 * q4 + 1] * sc);
-        const typename E::vec2 x1 = E::cvt2(dq[db][4 * q4 + 2] * sc, dq[db][4 * q4 + 3] * sc);
-        typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
-        *reinterpret_cast<typename E::vec4*>(drow + 32 * db + 8 * q4 + 4 * g) = x;
-      }
+  // the rows leave through LDS (store_rows_through_lds): every wave is done with the last tile first; a halved
+  // tile's writers use the part of LDS they have just read their partner's sums from
+  if (!halved) __syncthreads();
+  if (writer) {
+    char* patch = smem + (halved ? qc.rb * (16 * DBN * 64 * 4) : wave * row_patch_bytes<D>());
+    store_rows_through_lds<E, D, DBN>(patch, dq, a.scale, [&](const int r) -> T* {
+      const int rr = __shfl(row, r);
+      return rr >= 0 ? dqp + int64_t(rr) * a.dq_rs : nullptr;
+    });
   }
   FA_STAMP(g_trace_dq, 4, FA_CLOCK());
 }

@@ -469,21 +469,17 @@ void fwd_kernel(const KArgs a) {
     return;
   }
 
-  // epilogue: normalise, write O and LSE
+  // epilogue: normalise, write O and LSE (the rows leave through LDS, see store_rows_through_lds: every wave is
+  // done with the last tile first; a halved tile's writers use the part of LDS they have just read their partner's state from)
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  if (row >= 0 && writer) {
-    if (g == 0) lsep[row] = l_tot > 0.f ? m_ref + fast_log2(l_tot) : -INFINITY;
-    T* orow = op + int64_t(row) * a.o_rs;
-#pragma unroll
-    for (int db = 0; db < DBN; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
-        const typename E::vec2 x0 = E::cvt2(o[db][4 * q4 + 0] * inv, o[db][4 * q4 + 1] * inv);
-        const typename E::vec2 x1 = E::cvt2(o[db][4 * q4 + 2] * inv, o[db][4 * q4 + 3] * inv);
-        typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
-        *reinterpret_cast<typename E::vec4*>(orow + 32 * db + 8 * q4 + 4 * g) = x;
-      }
+  if (!halved) __syncthreads();
+  if (row >= 0 && writer && g == 0) lsep[row] = l_tot > 0.f ? m_ref + fast_log2(l_tot) : -INFINITY;
+  if (writer) {
+    char* patch = smem + (halved ? qc.rb * ((2 + 16 * DBN) * 64 * 4) : wave * row_patch_bytes<D>());
+    store_rows_through_lds<E, D, DBN>(patch, o, inv, [&](const int r) -> T* {
+      const int rr = __shfl(row, r);
+      return rr >= 0 ? op + int64_t(rr) * a.o_rs : nullptr;
+    });
   }
   FA_STAMP(g_trace_fwd, 4, FA_CLOCK());
 }

@@ -477,6 +477,42 @@ FA_DEV int split_range(const KArgs& a, const QWork& w, int& first, int& last) {
   return ns;
 }
 
+// A wave's 32 result rows on their way out.  The accumulators hold a row (or key) per lane and 4 consecutive
+// columns per register quad: stored from there, a wave instruction writes 64 pieces of 8 bytes, a row apart, and
+// every 128-byte line of the result fills up over sixteen instructions -- measured at 5-13 % of the id
+// workloads' kernel times.  So the rows pass through a patch of LDS that belongs to the wave (32 rows of
+// D * 2 + 16 bytes; LDS operations of one wave execute in issue order, so no barrier sits between the writes
+// and the reads) and leave as 16 bytes per lane, D / 8 lanes to a row: whole lines per instruction.
+// row_ptr(r) gives the address of row r of the wave (0..31) in memory, or nullptr for a row that does not exist.
+template <int D>
+constexpr int row_patch_bytes() { return 32 * (D * 2 + 16); }
+template <typename E, int D, int DBN, typename F>
+FA_DEV void store_rows_through_lds(char* patch, const f32x16 (&v)[DBN], const float sc, F&& row_ptr) {
+  using T = typename E::scalar;
+  using vec8 = typename E::vec8;
+  constexpr int PITCH = D * 2 + 16, CPR = D / 8, RPI = 64 / CPR, NI = 32 / RPI;
+  const int lane = threadIdx.x & 63, lq = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int db = 0; db < DBN; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      if (32 * db + 8 * q4 >= D) continue;  // padded columns of the D = 16 layout
+      const typename E::vec2 x0 = E::cvt2(v[db][4 * q4 + 0] * sc, v[db][4 * q4 + 1] * sc);
+      const typename E::vec2 x1 = E::cvt2(v[db][4 * q4 + 2] * sc, v[db][4 * q4 + 3] * sc);
+      typename E::vec4 x = {x0[0], x0[1], x1[0], x1[1]};
+      *reinterpret_cast<typename E::vec4*>(patch + lq * PITCH + (32 * db + 8 * q4 + 4 * g) * 2) = x;
+    }
+  asm volatile("" ::: "memory");   // (order only)
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int r = RPI * i + lane / CPR, cc = lane % CPR;
+    const vec8 x = *reinterpret_cast<const vec8*>(patch + r * PITCH + cc * 16);
+    T* p = row_ptr(r);
+    if (p != nullptr) *reinterpret_cast<vec8*>(p + cc * 8) = x;
+  }
+  asm volatile("" ::: "memory");
+}
+
 // Partial results travel between workgroups through device-scope accesses (they pass the
 // non-coherent cache levels access by access), so no cache-wide write-back or invalidate is needed.
 FA_DEV void store_dev(float* p, float x0, float x1) {
