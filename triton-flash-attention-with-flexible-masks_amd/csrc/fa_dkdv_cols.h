@@ -315,7 +315,7 @@ FA_DEV void dkdv_cols_body(const KArgs& a, const int bid, char* smem) {
             const vec8 x = *reinterpret_cast<const vec8*>(xp + kr * kXpPitch + cc * 16);
             const int key_o = nw + 16 * kh + kr;
             if (key_o < a.N && 32 * d0 + 8 * cc < D)
-              *reinterpret_cast<vec8*>(reinterpret_cast<char*>(obase) + ((unsigned)key_o * ors_b + (unsigned)(64 * d0 + 16 * cc))) = x;
+              __builtin_nontemporal_store(x, reinterpret_cast<vec8*>(reinterpret_cast<char*>(obase) + ((unsigned)key_o * ors_b + (unsigned)(64 * d0 + 16 * cc))));   // streaming: nobody reads these lines soon
           }
           asm volatile("" ::: "memory");   // the next writes to the patch are issued, hence executed, after these reads
         }
