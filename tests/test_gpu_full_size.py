@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests._tol import check_close
+from tests._tol import check_close, worst_ratio
 
 pytestmark = pytest.mark.gpu
 
@@ -90,14 +90,24 @@ def test_size_independent_properties(name):
     assert not torch.isnan(out2).any()
 
 
-# (batch, head) slices that meet the oracle, per configuration: the first and the last head of every batch
-# and further heads in between (cfg5: 16 slices, cfg3 and cfg4: 8), in groups that each stay well inside a minute
+# (batch, head) slices that meet the oracle, per configuration: every one of the 64 of cfg3 and cfg5, every other head
+# of cfg4 (the first and the last included; a slice of it keeps the host busy for seven seconds), in groups that each
+# stay well inside a minute
 SLICES = {
-    "cfg4_doc_causal_16k": [(0, 0), (0, 31), (0, 5), (0, 10), (0, 15), (0, 16), (0, 21), (0, 26)],
-    "cfg3_doc_causal_4k": [(0, 0), (0, 31), (1, 0), (1, 31), (0, 3), (0, 17), (1, 12), (1, 30)],
-    "cfg5_rect_fp16": [(b, h) for b in range(8) for h in (0, 7)],
+    "cfg4_doc_causal_16k": [(0, h) for h in (0, 31, 2, 4, 6, 8, 10, 12, 14, 16, 18, 20, 22, 24, 26, 28)],
+    "cfg3_doc_causal_4k": [(b, h) for b in range(2) for h in range(32)],
+    "cfg5_rect_fp16": [(b, h) for b in range(8) for h in range(8)],
 }
-_GROUP = {"cfg4_doc_causal_16k": 2, "cfg3_doc_causal_4k": 8, "cfg5_rect_fp16": 16}
+_GROUP = {"cfg4_doc_causal_16k": 4, "cfg3_doc_causal_4k": 32, "cfg5_rect_fp16": 32}
+# Per-element bound of the gradients (tests/_tol.py) times this, where the run over every slice needs it.  cfg3: its 64 slices
+# hold 100 million gradient elements; a dQ or dK element is a sum over up to 4096 products of a dS that was rounded to bf16
+# (flash_triton.py:306,417), and the tail of that error distribution reaches the bound of 2e-2.  Measured over the 64 slices
+# (seed 1): this library has one dQ element at 1.039 of the bound (slice (0,12)) and one dK element at 1.032 ((1,16)); the CPU
+# model of the reference's own storage roundings (oracle.attention_grads(store_dtype=bfloat16), result rounded too) has four
+# tensors over the bound on the same inputs, the worst at 1.142 (dK of slice (0,0)): no implementation that rounds where the
+# reference rounds meets the bound on every element here.  The ceilings sit just above what was measured; dV, O and LSE of
+# cfg3 and everything of cfg4 and cfg5 (fp16: 0.14 of the bound at most) are held to the plain bound.
+SLICE_CEILINGS = {"cfg3_doc_causal_4k": {"dq": 1.1, "dk": 1.1}}
 _gpu_results = {}
 
 
@@ -123,6 +133,7 @@ def test_slices_against_the_oracle(name, group):
     slices = SLICES[name][group * _GROUP[name]:(group + 1) * _GROUP[name]]
     print(f"case slices {name} {slices}", flush=True)
     assert w.H == w.Hk   # the configurations here are multi-head; dK / dV of a slice need no group sum
+    worst = {}
     for (b, h) in slices:
         sl = (slice(b, b + 1), slice(h, h + 1))
         ro, rl, rdq, rdk, rdv = O.attention_autograd(q[sl], k[sl], v[sl], do[sl], w.causal, None, eq[sl], ek[sl], 1)
@@ -132,7 +143,13 @@ def test_slices_against_the_oracle(name, group):
         assert (got_l[~dead] - rl[~dead]).abs().max().item() <= TOL_LSE
         assert (out[sl].float() - ro).abs().max().item() <= TOL_O
         for nm, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
-            check_close(f"{name} slice ({b},{h}) {nm}", got[sl], ref)
+            r, err, at = worst_ratio(got[sl], ref)
+            worst[nm] = max(worst.get(nm, 0.0), r)
+            if r > 0.9:
+                print(f"  {name} slice ({b},{h}) {nm}: worst err/bound {r:.3f} (err {err:.4g} at ref {at:.4g})", flush=True)
+            assert r <= SLICE_CEILINGS.get(name, {}).get(nm, 1.0), \
+                f"{name} slice ({b},{h}) {nm}: error {err:.5g} at reference value {at:.5g} is {r:.3f} x the bound"
+    print(f"  {name} group {group}: worst err/bound over {len(slices)} slices:", {n: round(r, 3) for n, r in worst.items()}, flush=True)
 
 
 def test_cfg2_plain_every_head_against_the_oracle():
